@@ -170,3 +170,120 @@ def read_config_json(model_dir: str) -> dict:
     if not isinstance(raw, dict):
         raise ConfigError(f"failed to parse {path}: top level is not an object")
     return raw
+
+
+# ---------------------------------------------------------------------------
+def _obj(raw: Mapping[str, Any], key: str, arch: str, where: str = "", optional: bool = False):
+    if key not in raw or raw[key] is None:
+        if optional:
+            return None
+        raise ConfigError(f"failed to parse {arch} config: missing required key `{where}{key}`")
+    if not isinstance(raw[key], dict):
+        raise ConfigError(f"failed to parse {arch} config: `{where}{key}` must be an object")
+    return raw[key]
+
+
+def _positive(raw: Mapping[str, Any], key: str, kind, arch: str, where: str):
+    try:
+        v = _get(raw, key, kind, arch)
+    except ConfigError as e:
+        raise ConfigError(str(e).replace(f"`{key}`", f"`{where}{key}`")) from None
+    if not v > 0:
+        raise ConfigError(f"failed to parse {arch} config: `{where}{key}` must be positive, got {v!r}")
+    return v
+
+
+@dataclasses.dataclass(frozen=True)
+class LatentMixerConfig:
+    heads: int
+    dim: int          # unrotated query/key dimensions a head
+    rot_dim: int      # rotated query/key dimensions a head (the key's are shared by all heads)
+    vdim: int         # value dimensions a head
+    kv_rank: int
+    q_rank: int
+    scale: float
+    rot_base: float
+    rot_dims: int     # how many of the rotated part's dimensions turn
+
+
+@dataclasses.dataclass(frozen=True)
+class LibodraMlpConfig:
+    kind: str                 # "dense" | "moe"
+    ff: int = 0               # dense: inner size; moe: an expert's inner size
+    limit: float = 0.0        # dense: the clamp
+    experts: int = 0
+    top: int = 0
+    shared_ff: int = 0        # moe: inner size of the shared expert, 0 = none
+
+
+@dataclasses.dataclass(frozen=True)
+class LibodraLayerConfig:
+    type: str
+    mixer: LatentMixerConfig
+    mlp: Optional[LibodraMlpConfig]
+
+
+@dataclasses.dataclass(frozen=True)
+class LibodraConfig:
+    """Libodra: a decoder of pre-norm layers listed one by one in ``layers``, each with a mixer that attends
+    through a latent (a learned sink in its softmax) and a feed-forward that is dense (clamped gated pair), a
+    mixture of experts chosen by token id from a table (with an optional shared expert), or absent.  Every size
+    and constant is read from here; there is no longest position and no end-of-sequence id."""
+    vocab: int
+    width: int
+    norm_eps: float
+    layers: Tuple[LibodraLayerConfig, ...]
+
+    ARCH = "Libodra"
+    MIXERS = ("latent_attention",)
+
+    @classmethod
+    def from_dict(cls, raw: Mapping[str, Any]) -> "LibodraConfig":
+        a = cls.ARCH
+        layers_raw = raw.get("layers")
+        if not isinstance(layers_raw, list) or not layers_raw:
+            raise ConfigError(f"failed to parse {a} config: `layers` must be a non-empty list")
+        layers = []
+        for i, lr in enumerate(layers_raw):
+            w = f"layers[{i}]."
+            if not isinstance(lr, dict):
+                raise ConfigError(f"failed to parse {a} config: `layers[{i}]` must be an object")
+            kind = _get(lr, "type", str, a)
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"failed to parse {a} config: `{w}type` {kind!r} is not one of {list(cls.MIXERS)}")
+            m = _obj(lr, "mixer", a, w)
+            mw = w + "mixer."
+            rot = _obj(m, "rot", a, mw)
+            rot_dim = _get(m, "rot_dim", int, a)
+            mixer = LatentMixerConfig(
+                heads=_positive(m, "heads", int, a, mw), dim=_positive(m, "dim", int, a, mw), rot_dim=rot_dim,
+                vdim=_positive(m, "vdim", int, a, mw), kv_rank=_positive(m, "kv_rank", int, a, mw),
+                q_rank=_positive(m, "q_rank", int, a, mw), scale=_positive(m, "scale", float, a, mw),
+                rot_base=_positive(rot, "base", float, a, mw + "rot."), rot_dims=_get(rot, "dims", int, a))
+            if mixer.rot_dims % 2 or mixer.rot_dims > mixer.rot_dim:
+                raise ConfigError(f"failed to parse {a} config: `{mw}rot.dims` ({mixer.rot_dims}) must be even and at "
+                                  f"most `rot_dim` ({mixer.rot_dim})")
+            f = _obj(lr, "mlp", a, w, optional=True)
+            mlp = None
+            if f is not None:
+                fw = w + "mlp."
+                fk = _get(f, "kind", str, a)
+                if fk == "dense":
+                    mlp = LibodraMlpConfig("dense", ff=_positive(f, "ff", int, a, fw), limit=_positive(f, "limit", float, a, fw))
+                elif fk == "moe":
+                    router = _obj(f, "router", a, fw)
+                    shared = _obj(f, "shared", a, fw, optional=True)
+                    mlp = LibodraMlpConfig(
+                        "moe", ff=_positive(_obj(f, "expert", a, fw), "ff", int, a, fw + "expert."),
+                        experts=_positive(router, "experts", int, a, fw + "router."),
+                        top=_positive(router, "top", int, a, fw + "router."),
+                        shared_ff=_positive(shared, "ff", int, a, fw + "shared.") if shared is not None else 0)
+                    if mlp.top > mlp.experts:
+                        raise ConfigError(f"failed to parse {a} config: `{fw}router.top` ({mlp.top}) exceeds "
+                                          f"`router.experts` ({mlp.experts})")
+                else:
+                    raise ConfigError(f"failed to parse {a} config: `{fw}kind` {fk!r} is not one of ['dense', 'moe']")
+            layers.append(LibodraLayerConfig(kind, mixer, mlp))
+        norm = _obj(raw, "norm", a)
+        return cls(vocab=_positive(raw, "vocab", int, a, ""), width=_positive(raw, "width", int, a, ""),
+                   norm_eps=_positive(norm, "eps", float, a, "norm."), layers=tuple(layers))

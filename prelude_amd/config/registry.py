@@ -70,6 +70,12 @@ def resolve_architecture(raw: Mapping[str, Any]) -> Architecture:
             a = _by_architecture_name(n)
             if a is not None:
                 return a
+    # a config that names its design plainly: `architecture`, the name as it stands
+    one = raw.get("architecture")
+    if isinstance(one, str):
+        for a in _ARCHS:
+            if _norm(one) in (_norm(x) for x in a.architecture_aliases):
+                return a
     mt = raw.get("model_type")
     if isinstance(mt, str):
         for a in _ARCHS:
@@ -77,4 +83,4 @@ def resolve_architecture(raw: Mapping[str, Any]) -> Architecture:
                 return a
     raise UnknownArchitecture(
         f"unable to resolve model architecture from config metadata: architectures={list(names)!r}, "
-        f"model_type={mt!r} (registered: {registered_architectures()})")
+        f"architecture={one!r}, model_type={mt!r} (registered: {registered_architectures()})")

@@ -157,6 +157,46 @@ int pa_logprobs(void* stream, const float* logits, const int* ids, float* lp, fl
 int pa_sample_wide(void* stream, const float* logits, const float* temperature, const int* top_k, const float* top_p,
                    const float* uniform, int* out, void* workspace, int rows, int vocab, int modes);
 
+// ---- a residual stream kept in 32-bit; activations the gated epilogues do not have (rowwise_wide.hip) ----
+// RMSNorm of x (+ residual): the residual is 32-bit and receives the unrounded sum (unless `rows`); x and out are of
+// `dtype`; x may be given as `slices` 32-bit partial sums [slices, rows, hidden] instead (then x is null).
+int pa_rmsnorm_wide(void* stream, int dtype, const void* x, const float* parts, int slices, long slice_stride,
+                    float* residual, const float* w, void* out, const int* rows, int nrows, int hidden, float eps);
+// gate_up [tokens, 2 inter], columns alternating gate_j, up_j -> out [tokens, inter]:
+// g = min(g, limit), u = clamp(u, -limit, limit), g * sigmoid(alpha g) * (u + 1)
+int pa_clamped_gate(void* stream, int dtype, const void* gate_up, void* out, int tokens, int inter, float limit, float alpha);
+// out = max(x, 0)^2
+int pa_relu_squared(void* stream, int dtype, const void* x, void* out, long total);
+
+// ---- attention through a latent (latent.hip) ----
+// in [tokens, q_rank + rank + rot]: cq_out [tokens, q_rank] = RMSNorm(first part) * wq; into the cache row slots[t]
+// ([rank + rot] elements a token): RMSNorm(second part) * wc, then the third part with its first rot_dims elements
+// rotated in pairs (2i, 2i+1) by the angle position * inv_freq[i].  slots null: nothing is cached.
+int pa_latent_prep(void* stream, int dtype, const void* in, const float* wq, const float* wc, const float* inv_freq,
+                   const int* positions, const int* slots, void* cq_out, void* cache, int tokens, int q_rank, int rank,
+                   int rot, int rot_dims, float eps);
+// in [tokens, heads, in_stride] -> out [tokens, heads, out_stride]: `width` elements from in_off to out_off of every
+// head, the first rot_dims of them rotated in pairs
+int pa_rotate_pairs(void* stream, int dtype, const void* in, void* out, const float* inv_freq, const int* positions,
+                    int tokens, int heads, int in_stride, int in_off, int out_stride, int out_off, int width, int rot_dims);
+// y[t, h, n] = sum_k x[t, h, k] wt[h, k, n]; strides in elements
+int pa_head_linear(void* stream, int dtype, const void* x, const void* wt, void* y, int tokens, int heads, int K, int N,
+                   long xs_t, long xs_h, long ys_t, long ys_h);
+// q [tokens, heads, rank + rot], cache [pages, page_size, rank + rot], sink [heads] or null -> out [tokens, heads, rank]
+int pa_latent_attn(void* stream, int dtype, const void* q, const void* cache, const float* sink, const int* block_table,
+                   int table_stride, const int* seq_of_token, const int* positions, void* out, int tokens, int nh, int rank,
+                   int rot, int page_size, int window, float scale);
+
+// ---- experts (moe.hip) ----
+int pa_moe_choices_by_table(void* stream, const int* ids, const int* table, int* choice, int tokens, int top, int vocab,
+                            int experts);
+int pa_moe_order(void* stream, const int* choice, int entries, int experts, int* counts, int* offsets, int* order, int* place);
+int pa_moe_linear(void* stream, int x_dtype, int w_dtype, int y_dtype, const void* x, const void* wt, void* y,
+                  const int* offsets, const int* order, int entries, int experts, int top, int K, int N, int from_tokens,
+                  int act);
+int pa_moe_combine(void* stream, int dtype, const float* y, const int* place, const float* weights, float weight,
+                   const void* base, void* out, int tokens, int top, int width);
+
 #ifdef __cplusplus
 }
 #endif

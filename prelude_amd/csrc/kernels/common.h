@@ -30,6 +30,14 @@ __device__ __forceinline__ float gate_activation(float x, int act) {
   return x / (1.0f + expf(-x));
 }
 
+// A gated pair with both halves clamped: g = min(g, limit), u = clamp(u, -limit, limit), and
+// g * sigmoid(alpha * g) * (u + 1); `limit` and `alpha` are the model's constants.
+__device__ __forceinline__ float clamped_gate(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+}
+
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(bf16 v) { return static_cast<float>(v); }
 template <typename T> __device__ __forceinline__ T from_f32(float v);

@@ -1036,3 +1036,213 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     check(kernels().pa_sample(_stream(), _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
                               _ptr(out), r, vocab))
     return out
+
+
+# ---------------------------------------------------------------------------
+# A residual stream kept in 32-bit
+def rmsnorm_wide(x, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None,
+                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``rmsnorm`` for a float32 residual [T, H] beside x [T, H] of the engine's type (or a ``SliceSums``): the sum
+    is taken and kept in 32-bit (the residual receives it unrounded, unless ``rows``), the output is of x's type."""
+    parts = x.parts if isinstance(x, SliceSums) else None
+    xt = None if parts is not None else x
+    _dev(xt, parts, weight, residual, rows)
+    _f32(weight, "norm weight")
+    _f32(residual, "residual")
+    m, h = x.shape
+    if weight.shape != (h,) or (residual is not None and tuple(residual.shape) != (m, h)):
+        raise NativeError(f"rmsnorm_wide: x {tuple(x.shape)} / weight {tuple(weight.shape)} / residual "
+                          f"{None if residual is None else tuple(residual.shape)}")
+    n = m
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.shape[0]
+    out = torch.empty((n, h), dtype=x.dtype, device=weight.device)
+    check(kernels().pa_rmsnorm_wide(_stream(), _CODES[x.dtype], _ptr(xt), _ptr(parts),
+                                    0 if parts is None else parts.shape[0], m * h, _ptr(residual), _ptr(weight), _ptr(out),
+                                    _ptr(rows), n, h, float(eps)))
+    return out
+
+
+def clamped_gate(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """gate_up [T, 2I] with columns alternating gate_j, up_j -> [T, I]: g = min(g, limit), u = clamp(u, -limit, limit),
+    g * sigmoid(alpha * g) * (u + 1), in 32-bit."""
+    _dev(gate_up)
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise NativeError(f"clamped_gate: input {tuple(gate_up.shape)} is not [T, 2I]")
+    inter = gate_up.shape[1] // 2
+    out = torch.empty((gate_up.shape[0], inter), dtype=gate_up.dtype, device=gate_up.device)
+    check(kernels().pa_clamped_gate(_stream(), _code(gate_up), _ptr(gate_up), _ptr(out), gate_up.shape[0], inter,
+                                    float(limit), float(alpha)))
+    return out
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    _dev(x)
+    out = torch.empty_like(x)
+    check(kernels().pa_relu_squared(_stream(), _code(x), _ptr(x), _ptr(out), x.numel()))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Attention through a latent
+def latent_prep(down: torch.Tensor, q_weight: torch.Tensor, c_weight: torch.Tensor, inv_freq: Optional[torch.Tensor],
+                positions: torch.Tensor, slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], q_rank: int,
+                rank: int, rot: int, rot_dims: int, eps: float) -> torch.Tensor:
+    """The merged down projection [T, q_rank + rank + rot]: returns the normed query latent [T, q_rank]; writes the
+    normed latent and the rotated shared key part of every token into ``cache`` [pages, page, rank + rot] at ``slots``."""
+    _dev(down, q_weight, c_weight, inv_freq, positions, slots, cache)
+    _f32(q_weight, "query latent norm weight")
+    _f32(c_weight, "latent norm weight")
+    _f32(inv_freq, "rotary frequencies")
+    _i32(positions, "positions")
+    t = down.shape[0]
+    if down.dim() != 2 or down.shape[1] != q_rank + rank + rot or q_weight.shape != (q_rank,) or c_weight.shape != (rank,):
+        raise NativeError(f"latent_prep: input {tuple(down.shape)} for parts {q_rank} + {rank} + {rot}")
+    if positions.shape != (t,) or (rot_dims and (inv_freq is None or inv_freq.shape != (rot_dims // 2,))):
+        raise NativeError("latent_prep: positions or rotary frequencies do not match")
+    if slots is not None:
+        _i32(slots, "slots")
+        if slots.shape != (t,) or cache is None or cache.dim() != 3 or cache.shape[2] != rank + rot or cache.dtype != down.dtype:
+            raise NativeError(f"latent_prep: cache must be [pages, page, {rank + rot}] of {down.dtype}")
+    cq = torch.empty((t, q_rank), dtype=down.dtype, device=down.device)
+    check(kernels().pa_latent_prep(_stream(), _code(down), _ptr(down), _ptr(q_weight), _ptr(c_weight), _ptr(inv_freq),
+                                   _ptr(positions), _ptr(slots), _ptr(cq), _ptr(cache) if slots is not None else None, t,
+                                   q_rank, rank, rot, rot_dims, float(eps)))
+    return cq
+
+
+def rotate_pairs(x: torch.Tensor, out: torch.Tensor, inv_freq: Optional[torch.Tensor], positions: torch.Tensor, in_off: int,
+                 out_off: int, width: int, rot_dims: int) -> None:
+    """x [T, heads, a] -> out [T, heads, b]: ``width`` elements from ``in_off`` of every head to ``out_off``, the first
+    ``rot_dims`` of them rotated in pairs (2i, 2i+1) by position * inv_freq[i]."""
+    _dev(x, out, inv_freq, positions)
+    _f32(inv_freq, "rotary frequencies")
+    _i32(positions, "positions")
+    if x.dim() != 3 or out.dim() != 3 or x.shape[:2] != out.shape[:2] or x.dtype != out.dtype or positions.shape != (x.shape[0],):
+        raise NativeError(f"rotate_pairs: x {tuple(x.shape)} / out {tuple(out.shape)}")
+    if rot_dims and (inv_freq is None or inv_freq.shape != (rot_dims // 2,)):
+        raise NativeError("rotate_pairs: rotary frequencies do not match the rotated width")
+    check(kernels().pa_rotate_pairs(_stream(), _code(x), _ptr(x), _ptr(out), _ptr(inv_freq), _ptr(positions), x.shape[0],
+                                    x.shape[1], x.shape[2], int(in_off), out.shape[2], int(out_off), int(width), int(rot_dims)))
+
+
+def head_linear(x: torch.Tensor, wt: torch.Tensor, out: torch.Tensor, k: int, n: int, x_off: int = 0, out_off: int = 0) -> None:
+    """out[t, h, out_off : out_off + n] = W[h] x[t, h, x_off : x_off + k] for x [T, heads, a], out [T, heads, b] and the
+    weight as ``wt`` [heads, k, n] (the transposes of the heads' matrices)."""
+    _dev(x, wt, out)
+    if (x.dim() != 3 or out.dim() != 3 or x.shape[:2] != out.shape[:2] or tuple(wt.shape) != (x.shape[1], k, n)
+            or not (x.dtype == wt.dtype == out.dtype) or x_off + k > x.shape[2] or out_off + n > out.shape[2]):
+        raise NativeError(f"head_linear: x {tuple(x.shape)} / wt {tuple(wt.shape)} / out {tuple(out.shape)}")
+    el = x.element_size()
+    check(kernels().pa_head_linear(_stream(), _code(x), x.data_ptr() + x_off * el, _ptr(wt), out.data_ptr() + out_off * el,
+                                   x.shape[0], x.shape[1], int(k), int(n), x.shape[1] * x.shape[2], x.shape[2],
+                                   out.shape[1] * out.shape[2], out.shape[2]))
+
+
+def latent_attention_generic(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], block_table: torch.Tensor,
+                             seq_of_token: torch.Tensor, positions: torch.Tensor, rank: int, window: int,
+                             scale: float) -> torch.Tensor:
+    """Causal attention of q [T, heads, rank + rot] over cached latents [pages, page, rank + rot] (the value of a key
+    is its first ``rank`` elements), with ``sink`` [heads] joining each head's softmax denominator as exp(sink_h);
+    returns [T, heads, rank].  32-bit arithmetic; any mix of portions and single tokens."""
+    _dev(q, cache, sink, block_table, seq_of_token, positions)
+    _f32(sink, "sink")
+    _i32(block_table, "block_table")
+    _i32(seq_of_token, "seq_of_token")
+    _i32(positions, "positions")
+    t, nh, dk = q.shape
+    if cache.dim() != 3 or cache.shape[2] != dk or cache.dtype != q.dtype or not 0 < rank <= dk:
+        raise NativeError(f"latent_attention: q {tuple(q.shape)} / cache {tuple(cache.shape)} / rank {rank}")
+    if seq_of_token.shape != (t,) or positions.shape != (t,) or block_table.dim() != 2 or (sink is not None and sink.shape != (nh,)):
+        raise NativeError("latent_attention: index arrays or sinks do not match")
+    out = torch.empty((t, nh, rank), dtype=q.dtype, device=q.device)
+    check(kernels().pa_latent_attn(_stream(), _code(q), _ptr(q), _ptr(cache), _ptr(sink), _ptr(block_table),
+                                   block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out), t, nh, int(rank),
+                                   dk - int(rank), cache.shape[1], int(window), float(scale)))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Experts
+class ExpertOrder:
+    """A step's (token, choice) entries put in the order of their experts: ``offsets`` [E + 1], ``order`` [entries]
+    (position -> entry), ``place`` [entries] (entry -> position), all int32 on the device."""
+
+    def __init__(self, offsets, order, place, entries: int, experts: int, top: int):
+        self.offsets, self.order, self.place = offsets, order, place
+        self.entries, self.experts, self.top = entries, experts, top
+
+
+def moe_choices_by_table(token_ids: torch.Tensor, table: torch.Tensor, experts: int) -> torch.Tensor:
+    """choice[t * top + j] = table[token_ids[t], j]: experts by token id, no router."""
+    _dev(token_ids, table)
+    _i32(token_ids, "token ids")
+    _i32(table, "expert table")
+    if token_ids.dim() != 1 or table.dim() != 2:
+        raise NativeError(f"moe_choices_by_table: ids {tuple(token_ids.shape)} / table {tuple(table.shape)}")
+    t, top = token_ids.shape[0], table.shape[1]
+    choice = torch.empty(t * top, dtype=torch.int32, device=table.device)
+    check(kernels().pa_moe_choices_by_table(_stream(), _ptr(token_ids), _ptr(table), _ptr(choice), t, top, table.shape[0],
+                                            int(experts)))
+    return choice
+
+
+def moe_order(choice: torch.Tensor, experts: int, top: int) -> ExpertOrder:
+    _dev(choice)
+    _i32(choice, "choices")
+    n = choice.shape[0]
+    ints = torch.empty(2 * experts + 1 + 2 * n, dtype=torch.int32, device=choice.device)
+    counts, offsets = ints[:experts], ints[experts: 2 * experts + 1]
+    order, place = ints[2 * experts + 1: 2 * experts + 1 + n], ints[2 * experts + 1 + n:]
+    check(kernels().pa_moe_order(_stream(), _ptr(choice), n, int(experts), _ptr(counts), _ptr(offsets), _ptr(order), _ptr(place)))
+    return ExpertOrder(offsets, order, place, n, int(experts), int(top))
+
+
+def moe_linear(x: torch.Tensor, wt: torch.Tensor, eo: ExpertOrder, from_tokens: bool, relu_squared_epilogue: bool = False,
+               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y[p] = act(W[expert of p] x[row of p]) over the ordered positions p; ``wt`` [E, k, n] (the experts' matrices
+    transposed); ``from_tokens``: x holds a row per token (position p reads its token's), else a row per position."""
+    _dev(x, wt)
+    e, k, n = wt.shape
+    rows = eo.entries // eo.top if from_tokens else eo.entries
+    if x.dim() != 2 or tuple(x.shape) != (rows, k) or e != eo.experts or x.dtype != wt.dtype:
+        raise NativeError(f"moe_linear: x {tuple(x.shape)} {x.dtype} / wt {tuple(wt.shape)} {wt.dtype} for {eo.entries} entries")
+    out_dtype = out_dtype or x.dtype
+    y = torch.empty((eo.entries, n), dtype=out_dtype, device=x.device)
+    check(kernels().pa_moe_linear(_stream(), _code(x), _code(wt), _CODES[out_dtype], _ptr(x), _ptr(wt), _ptr(y), _ptr(eo.offsets),
+                                  _ptr(eo.order), eo.entries, eo.experts, eo.top, k, n, 1 if from_tokens else 0,
+                                  1 if relu_squared_epilogue else 0))
+    return y
+
+
+def moe_combine(y: torch.Tensor, eo: ExpertOrder, weight: float, base: Optional[torch.Tensor], out_dtype: torch.dtype,
+                weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = base[t] + sum_j w * y[place[t * top + j]] in ascending j; y float32 [entries, H]; ``weights`` float32
+    [entries] per entry, else ``weight`` for all."""
+    _dev(y, base, weights)
+    _f32(y, "expert outputs")
+    _f32(weights, "entry weights")
+    t = eo.entries // eo.top
+    h = y.shape[1]
+    if y.shape[0] != eo.entries or (base is not None and (tuple(base.shape) != (t, h) or base.dtype != out_dtype)):
+        raise NativeError(f"moe_combine: y {tuple(y.shape)} / base {None if base is None else tuple(base.shape)}")
+    out = torch.empty((t, h), dtype=out_dtype, device=y.device)
+    check(kernels().pa_moe_combine(_stream(), _CODES[out_dtype], _ptr(y), _ptr(eo.place), _ptr(weights), float(weight), _ptr(base),
+                                   _ptr(out), t, eo.top, h))
+    return out
+
+
+LATENT_MAX_WIDTH = 1024   # rank + rot of a cached latent vector the attention kernels take
+
+
+def latent_attention(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], group, step, rank: int,
+                     window: int, scale: float) -> torch.Tensor:
+    """Attention of one step over a cache of latents; picks the kernel for the sizes at hand (``group``: the
+    step's ``GroupStep`` of the cache group, ``step``: the ``StepBatch``)."""
+    return latent_attention_generic(q, cache, sink, group.block_table, step.seq_of_token, step.positions, rank, window, scale)
+
+
+def linear_clamped_gate(x: torch.Tensor, w, limit: float, alpha: float) -> torch.Tensor:
+    """The clamped gated pair of ``clamped_gate`` over x W^T for a weight [2I, K] whose rows alternate gate_j, up_j."""
+    return clamped_gate(linear(x, w), limit, alpha)

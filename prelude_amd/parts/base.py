@@ -17,7 +17,8 @@ Categories and the interface each must have:
               ``SlotCacheSpec`` (``StateSpec``) | ``None``;
               ``forward(x, step, cache, write_cache=True)``
 ``ffn``       ``forward(x)``; ``forward_after_norm(x, residual, norm) -> (residual, out)`` (given by the base class:
-              the norm's ``forward_residual``, then ``forward``) is what a block calls behind its mixer
+              the norm's ``forward_residual``, then ``forward``) is what a block calls behind its mixer; one that
+              says ``NEEDS_STEP`` gets the step too (``step=``), to choose experts by token id, say
 ``block``     ``forward(hidden, residual, step, cache, write_cache) -> (hidden, residual)``
 ``embedding`` ``forward(token_ids)``
 ``head``      ``forward(hidden_rows) -> float32 logits``
@@ -37,12 +38,14 @@ import torch
 MATRIX = "matrix"   # engine element type; N(0, std)
 VECTOR = "vector"   # float32; N(0, std)            (biases)
 NORM = "norm"       # float32; 1 + N(0, norm_std)   (norm scales)
+TABLE = "table"     # int32; every row distinct integers below ``TensorReq.high``   (lookup tables)
 
 
 @dataclasses.dataclass(frozen=True)
 class TensorReq:
     shape: Tuple[int, ...]
     kind: str = MATRIX
+    high: int = 0       # TABLE: entries are integers in [0, high)
 
 
 class PagedCacheSpec:
@@ -139,6 +142,30 @@ class KVCacheSpec(PagedCacheSpec):
                             group)
 
 
+@dataclasses.dataclass
+class LatentLayerCache:
+    """What a mixer that attends through a latent gets: one vector a token, in pages."""
+    latent: torch.Tensor   # [pages, page_size, rank + rot]
+    group: int
+
+
+@dataclasses.dataclass(frozen=True)
+class LatentCacheSpec(PagedCacheSpec):
+    """One vector per token, in pages: a latent of ``rank`` elements that stands for the keys and values of all
+    heads, followed by ``rot`` elements of a rotated key part the heads share.  Layout per cache slot
+    ``[pages, page_size, rank + rot]``: a token's vector is one run of memory, read whole for a score and by its
+    first ``rank`` elements as the value."""
+    rank: int
+    rot: int
+    window: int = 0
+
+    def bytes_per_token(self, element_size: int) -> int:
+        return (self.rank + self.rot) * element_size
+
+    def allocate(self, pages, page_size, dtype, device, group):
+        return LatentLayerCache(torch.zeros((pages, page_size, self.rank + self.rot), dtype=dtype, device=device), group)
+
+
 @dataclasses.dataclass(frozen=True)
 class StateSpec(SlotCacheSpec):
     """State of fixed size per request: name -> (shape, element type).  Zeroed when a request starts."""
@@ -201,10 +228,14 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    # True for a feed-forward that reads the step itself (its token ids, say, to choose experts by): ``forward`` and
+    # ``forward_after_norm`` are then called with ``step=`` the ``StepBatch``.
+    NEEDS_STEP = False
+
+    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
         raise NotImplementedError
 
-    def forward_after_norm(self, x, residual, norm: "Norm"):
+    def forward_after_norm(self, x, residual, norm: "Norm", step=None):
         """(new residual, forward(norm of residual + x)): what a block asks for behind a mixer.  A feed-forward whose
         first kernel can take the add and the norm in (it learns the norm's kind from ``norm.as_rms()``) does so
         here; this is the plain order."""
@@ -212,7 +243,7 @@ class FeedForward(Part):
             from ..ops.kernels import as_tensor
             x = as_tensor(x)
         residual, h = norm.forward_residual(x, residual)
-        return residual, self.forward(h)
+        return residual, (self.forward(h, step=step) if self.NEEDS_STEP else self.forward(h))
 
 
 class Norm(Part):

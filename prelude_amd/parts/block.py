@@ -27,5 +27,25 @@ class PreNormBlock(Block):
             hidden = K.as_tensor(hidden)
         residual, h = self.input_norm.forward_residual(hidden, residual)
         h = self.mixer.forward(h, step, cache, write_cache)
-        residual, h = self.ffn.forward_after_norm(h, residual, self.post_mixer_norm)
+        if getattr(self.ffn, "NEEDS_STEP", False):
+            residual, h = self.ffn.forward_after_norm(h, residual, self.post_mixer_norm, step=step)
+        else:
+            residual, h = self.ffn.forward_after_norm(h, residual, self.post_mixer_norm)
         return h, residual
+
+
+@register_part("block", "prenorm_mixer_only")
+class PreNormMixerBlock(Block):
+    """A layer without a feed-forward: norm -> mixer, the add deferred into the next norm as in ``prenorm``."""
+    GRAPH_SAFE_PORTIONS = True
+
+    SLOTS = {"input_norm": "norm", "mixer": "mixer"}
+
+    def __init__(self, input_norm, mixer):
+        self.input_norm, self.mixer = input_norm, mixer
+
+    def forward(self, hidden, residual, step, cache, write_cache=True):
+        if not self.input_norm.TAKES_SLICE_SUMS:
+            hidden = K.as_tensor(hidden)
+        residual, h = self.input_norm.forward_residual(hidden, residual)
+        return self.mixer.forward(h, step, cache, write_cache), residual

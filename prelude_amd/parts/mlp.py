@@ -52,3 +52,32 @@ class GatedMLP(FeedForward):
             return super().forward_after_norm(x, residual, norm)
         residual, h = K.linear_gated_after_norm(x, residual, rms[0], rms[1], self.gate_up, self.activation)
         return residual, K.linear(h, self.down, slices_ok=True)
+
+
+@register_part("ffn", "clamped_gated_mlp")
+class ClampedGatedMLP(FeedForward):
+    """down(y) with g = min(gate(x), limit), u = clamp(up(x), -limit, limit), y = g * sigmoid(alpha * g) * (u + 1);
+    ``limit`` and ``alpha`` are the model's constants.  Gate and up are one matrix with alternating rows, as in
+    ``gated_mlp``; the activation is computed in 32-bit from the product's pairs."""
+    LAUNCHES = 3
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702):
+        if not limit > 0:
+            raise PartError(f"clamped_gated_mlp: a limit of {limit} is not positive")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.gate_up = None
+        self.down = None
+
+    def tensors(self):
+        h, i = self.hidden_size, self.intermediate_size
+        return {"gate": TensorReq((i, h), MATRIX), "up": TensorReq((i, h), MATRIX), "down": TensorReq((h, i), MATRIX)}
+
+    def load(self, tensors, dtype, device):
+        self.gate_up = K.prepare_weight(torch.stack([tensors["gate"], tensors["up"]], dim=1)
+                                        .reshape(2 * self.intermediate_size, self.hidden_size).contiguous())
+        self.down = K.prepare_weight(tensors["down"])
+
+    def forward(self, x):
+        return K.linear(K.linear_clamped_gate(x, self.gate_up, self.limit, self.alpha), self.down, slices_ok=True)

@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 
 from ..ops import kernels as K
-from .base import NORM, Norm, TensorReq, register_part
+from .base import NORM, VECTOR, Norm, PartError, TensorReq, register_part
 
 
 @register_part("norm", "rms_norm")
@@ -21,16 +21,23 @@ class RMSNorm(Norm):
 
     TAKES_SLICE_SUMS = True
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, weight_offset: float = 0.0, residual_float32: bool = False):
+        """``weight_offset``: the stored weight lies around zero and the gain is ``offset + weight`` (added once,
+        in 32-bit, when the weight is loaded).  ``residual_float32``: the residual stream this norm adds to is
+        kept in 32-bit whatever the engine's element type; the normed output is of the engine's type."""
         self.size = int(size)
         self.eps = float(eps)
+        self.weight_offset = float(weight_offset)
+        self.residual_float32 = bool(residual_float32)
         self.weight: Optional[torch.Tensor] = None
 
     def tensors(self):
-        return {"weight": TensorReq((self.size,), NORM)}
+        # a weight stored around zero is drawn around zero in the random-weights mode too
+        return {"weight": TensorReq((self.size,), VECTOR if self.weight_offset else NORM)}
 
     def load(self, tensors, dtype, device):
-        self.weight = tensors["weight"]
+        w = tensors["weight"]
+        self.weight = (w + self.weight_offset).contiguous() if self.weight_offset else w
 
     def as_rms(self):
         return self.weight, self.eps
@@ -43,9 +50,18 @@ class RMSNorm(Norm):
         residual is updated in place with residual + x."""
         if residual is None:
             x = K.as_tensor(x)
+            if self.residual_float32:
+                # the stream starts as a 32-bit copy of x (x itself when the engine's type is 32-bit already)
+                return K.to_f32(x), K.rmsnorm(x, self.weight, self.eps)
             return x, K.rmsnorm(x, self.weight, self.eps)
+        if self.residual_float32:
+            if residual.dtype != torch.float32:
+                raise PartError("rms_norm: a norm with a 32-bit residual was handed one of another type")
+            return residual, K.rmsnorm_wide(x, self.weight, self.eps, residual=residual)
         out = K.rmsnorm(x, self.weight, self.eps, residual=residual)
         return residual, out
 
     def forward_rows(self, x, residual, rows):
+        if self.residual_float32 and residual is not None:
+            return K.rmsnorm_wide(x, self.weight, self.eps, residual=residual, rows=rows)
         return K.rmsnorm(x, self.weight, self.eps, residual=residual, rows=rows)

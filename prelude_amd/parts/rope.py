@@ -35,3 +35,25 @@ class RotaryEmbedding(PositionEncoding):
         ang = pos * inv_freq.reshape(1, -1)
         self.cos = torch.cos(ang).contiguous().to(device)
         self.sin = torch.sin(ang).contiguous().to(device)
+
+
+@register_part("position", "rotary_frequencies")
+class RotaryFrequencies(PositionEncoding):
+    """The frequencies alone, f_i = theta^(-2i/d) for i < d/2 (the power in 64-bit, rounded once to 32-bit): the
+    mixers' kernels take the angle position * f_i and its cosine and sine themselves, in 32-bit, so there is no
+    table and no longest position.  How the rotated dimensions are paired is the mixer's business."""
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, rotary_dim: int, theta: float):
+        if rotary_dim <= 0 or rotary_dim % 2:
+            raise PartError(f"rotary_frequencies: rotary width {rotary_dim} must be positive and even")
+        if theta <= 0:
+            raise PartError(f"rotary_frequencies: base {theta} must be positive")
+        self.rotary_dim = int(rotary_dim)
+        self.theta = float(theta)
+        self.inv_freq: Optional[torch.Tensor] = None
+
+    def prepare(self, device):
+        d = self.rotary_dim
+        i = torch.arange(0, d // 2, dtype=torch.float64)
+        self.inv_freq = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / d).to(torch.float32).to(device)

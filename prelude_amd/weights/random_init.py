@@ -30,7 +30,7 @@ from typing import Any, Mapping
 import torch
 
 from ..config.registry import resolve_architecture
-from ..parts.base import MATRIX, NORM
+from ..parts.base import MATRIX, NORM, TABLE
 from .safetensors_io import write_safetensors
 
 
@@ -72,9 +72,19 @@ def _draw(name: str, req, seed: int, std: float, norm_std: float, device: torch.
     n = 1
     for d in req.shape:
         n *= int(d)
+    if req.kind == TABLE:
+        # every row a draw of distinct integers below ``high``: the places of the row's smallest variates
+        rows, top = int(req.shape[0]), int(req.shape[1])
+        z = _standard_normal(rows * int(req.high), _seed_for(seed, name), device).reshape(rows, int(req.high))
+        return torch.argsort(z, dim=1, stable=True)[:, :top].to(torch.int32).contiguous()
     t = _standard_normal(n, _seed_for(seed, name), device).reshape(req.shape)
     # one multiplication, then (for norm scales) one addition: separate steps, so no device contracts them
     return t.mul_(norm_std).add_(1.0) if req.kind == NORM else t.mul_(std)
+
+
+def _kept_as(req, dtype: torch.dtype) -> torch.dtype:
+    """The element type a part receives a tensor of this kind in."""
+    return dtype if req.kind == MATRIX else (torch.int32 if req.kind == TABLE else torch.float32)
 
 
 def random_tensors(raw_config: Mapping[str, Any], seed: int, std: float = 0.02, norm_std: float = 0.01,
@@ -87,7 +97,7 @@ def random_tensors(raw_config: Mapping[str, Any], seed: int, std: float = 0.02, 
     if device is None:
         device = "cuda" if torch.cuda.is_available() else "cpu"
     device = torch.device(device)
-    return {name: _draw(name, req, seed, std, norm_std, device).to(dtype).cpu()
+    return {name: _draw(name, req, seed, std, norm_std, device).to(torch.int32 if req.kind == TABLE else dtype).cpu()
             for name, req in model.tensor_requests().items()}
 
 
@@ -110,7 +120,7 @@ def load_random(model, dtype: torch.dtype, device: torch.device, seed: int = 0, 
     cache = {}
 
     def fetch(name: str, req):
-        want = dtype if req.kind == MATRIX else torch.float32
+        want = _kept_as(req, dtype)
         key = (name, want)
         if key not in cache:      # a tensor named twice (a tied head) is drawn once and shared
             cache[key] = _draw(name, req, seed, std, norm_std, device).to(want).contiguous()
@@ -127,5 +137,5 @@ def random_tensors_on_device(raw_config: Mapping[str, Any], seed: int, device, s
     arch = resolve_architecture(raw_config)
     model = CausalLM(arch.build_spec(arch.parse_config(raw_config)))
     device = torch.device(device)
-    return {name: _draw(name, req, seed, std, norm_std, device).to(dtype if req.kind == MATRIX else torch.float32)
+    return {name: _draw(name, req, seed, std, norm_std, device).to(_kept_as(req, dtype))
             for name, req in model.tensor_requests().items()}
