@@ -76,6 +76,9 @@ _KERNEL_API = {
     "pa_rotate_pairs": (I, [P, I, P, P, P, P, I, I, I, I, I, I, I, I]),
     "pa_head_linear": (I, [P, I, P, P, P, I, I, I, I, c_long, c_long, c_long, c_long]),
     "pa_latent_attn": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
+    "pa_latent_attn_mfma_supports": (I, [I, I, I]),
+    "pa_latent_attn_mfma_workspace": (c_long, [I, I, I, I]),
+    "pa_latent_attn_mfma": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I]),
     "pa_moe_choices_by_table": (I, [P, P, P, P, I, I, I, I]),
     "pa_moe_order": (I, [P, P, I, I, P, P, P, P]),
     "pa_moe_linear": (I, [P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I]),

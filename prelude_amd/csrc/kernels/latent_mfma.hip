@@ -1,0 +1,321 @@
+// Attention over a cache of latents on the matrix cores (bfloat16 in, 32-bit scores, softmax and sums).
+//
+// All heads read the same cached vectors, so the rows of the score matrix are (token, head) pairs: a workgroup
+// of four wavefronts owns 64 consecutive rows of one sequence's portion (row = token * heads + head), 16 a
+// wavefront, and walks the keys in blocks of 32.  A block is brought into LDS once per workgroup: the vectors as
+// they lie in the cache (rows of rank + rot elements, the score's operand), and the first `rank` elements of each
+// again transposed ([element][key]: the operand of the weighted sum, whose contraction runs over keys).
+//
+//   S^T = K Q^T     A = 16 keys x 32 elements from LDS, B = the wavefront's queries, kept in registers
+//   O^T = V^T P^T   A = 16 elements x 32 keys from the transposed copy, B = the probabilities just computed
+//
+// v_mfma_f32_16x16x32_bf16 (lane l, g = l / 16, r = l % 16): A row r, columns 8g..8g+7; B column r, rows 8g..8g+7;
+// C column r, rows 4g..4g+3.  A block's 32 keys are two score tiles; row 4a + i of tile t stands for key
+// 8a + 4t + i, so lane group g ends up with the scores of keys 8g..8g+7 of its query: packed, they are the B
+// operand of the second product as they stand.
+//
+// Few rows a sequence (single decoded tokens) would leave the chip empty: then the keys are cut into splits of
+// `split_keys` (grid.z), each leaving an unnormalised partial (maximum, sum, weighted sum) that a merge kernel adds
+// up in split order.  The sink joins last, as one more term exp(sink_h) of the denominator.
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+constexpr float kLog2eL = 1.4426950408889634f;
+constexpr int kLmRows = 64;      // query rows a workgroup
+constexpr int kLmKeys = 32;      // keys a block
+constexpr int kLmPad = 8;        // elements of padding behind an LDS row
+
+__device__ __forceinline__ f32x4 mfma16l(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// RT: value tiles of 16 elements held in registers (rank <= 16 RT); QS: steps of 32 elements of a query held in
+// registers (rank + rot <= 32 QS).
+template <int RT, int QS>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ cache, const float* __restrict__ sink,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
+    float* __restrict__ ws, int nh, int rank, int rot, int page_size, int window, float scale, int split_keys,
+    int n_splits) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int dk = rank + rot;
+  const int dk_steps = (dk + 31) / 32;
+  const int k_stride = dk_steps * 32 + kLmPad;                 // elements
+  const int v_tiles = (rank + 15) / 16;
+  constexpr int v_stride = kLmKeys + kLmPad;
+  bf16* k_lds = reinterpret_cast<bf16*>(lds_raw);              // [32][k_stride]
+  bf16* v_lds = k_lds + kLmKeys * k_stride;                    // [v_tiles * 16][v_stride]
+
+  const int seq = seq_ids ? seq_ids[blockIdx.y] : blockIdx.y;
+  const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
+  const int rows = qn * nh;
+  const int rb = blockIdx.x * kLmRows;
+  if (rb >= rows) return;
+  const int ctx = context_lens[seq];
+  const int p0 = ctx - qn;                                     // position of the portion's first token
+  const int* table = block_table + (size_t)seq * table_stride;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+
+  // this lane's query row (clamped: rows past the end repeat the last one and are not stored)
+  const int row = rb + wave * 16 + r;
+  const bool row_ok = row < rows;
+  const int rowc = row_ok ? row : rows - 1;
+  const int tq = rowc / nh, head = rowc % nh;
+  const int pos = p0 + tq;
+  const int lo_row = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+
+  // keys the workgroup walks: up to its last row's position, from its first row's window edge, inside its split
+  const int last_row = (rb + kLmRows - 1 < rows ? rb + kLmRows - 1 : rows - 1);
+  const int hi_wg = p0 + last_row / nh;
+  const int first_pos = p0 + rb / nh;
+  int lo_wg = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+  int end_wg = hi_wg + 1;
+  if (n_splits > 1) {
+    const int s0 = blockIdx.z * split_keys;
+    lo_wg = lo_wg > s0 ? lo_wg : s0;
+    end_wg = end_wg < s0 + split_keys ? end_wg : s0 + split_keys;
+  }
+  lo_wg = (lo_wg / kLmKeys) * kLmKeys;                         // blocks stand at multiples of 32 keys
+
+  // queries: B operand, column r = this lane's row, rows 8g..8g+7 of every step of 32 elements
+  bf16x8 qf[QS];
+  {
+    const bf16* qr = q + ((size_t)(q0 + tq) * nh + head) * dk;
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+      const int d = 32 * s + 8 * g;
+      bf16x8 v = {};
+      if (d + 8 <= dk) v = *reinterpret_cast<const bf16x8*>(qr + d);
+      qf[s] = v;
+    }
+  }
+  f32x4 o[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const float c = scale * kLog2eL;
+  const int chunks = dk_steps * 4;                             // 16-byte pieces of a staged row
+
+  for (int b0 = lo_wg; b0 < end_wg; b0 += kLmKeys) {
+    __syncthreads();
+    // ---- stage the block: rows as they are, and their first `rank` elements transposed ----
+    // (neighbouring threads take neighbouring keys, so that the transposed 2-byte stores of a wavefront fall into
+    // one row of the copy instead of into rows a multiple of 32 banks apart)
+    for (int i = threadIdx.x; i < kLmKeys * chunks; i += 256) {
+      const int key = i % kLmKeys, ch = i / kLmKeys;
+      const int kidx = b0 + key;
+      bf16x8 v = {};
+      if (kidx < end_wg && 8 * ch + 8 <= dk) {
+        const int page = table[kidx / page_size];
+        if (page >= 0) v = *reinterpret_cast<const bf16x8*>(cache + ((size_t)page * page_size + kidx % page_size) * dk + 8 * ch);
+      }
+      *reinterpret_cast<bf16x8*>(k_lds + key * k_stride + 8 * ch) = v;
+      if (8 * ch < v_tiles * 16) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v_lds[(8 * ch + j) * v_stride + key] = (8 * ch + j < rank) ? v[j] : (bf16)0.f;
+      }
+    }
+    __syncthreads();
+    // ---- scores of 32 keys for this wavefront's 16 rows ----
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16* kr = k_lds + (8 * (r / 4) + 4 * t + (r % 4)) * k_stride + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < QS; ++ks) {
+        if (ks < dk_steps) s[t] = mfma16l(*reinterpret_cast<const bf16x8*>(kr + 32 * ks), qf[ks], s[t]);
+      }
+    }
+    // ---- mask, running maximum, probabilities ----
+    float bm = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int kidx = b0 + 8 * g + 4 * t + i;
+        const bool ok = kidx <= pos && kidx >= lo_row && kidx < end_wg;
+        s[t][i] = ok ? s[t][i] : -INFINITY;
+        bm = fmaxf(bm, s[t][i]);
+      }
+    bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
+    bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
+    const float m_new = fmaxf(m, bm);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f((m - m_use) * c);
+    float psum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = exp2f((s[t][i] - m_use) * c);       // exp2(-inf) = 0 for masked keys
+        psum += p;
+        pf[4 * t + i] = (bf16)p;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    // ---- weighted sum: O^T += V^T P^T ----
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      if (t < v_tiles) {
+        o[t] *= alpha;
+        o[t] = mfma16l(*reinterpret_cast<const bf16x8*>(v_lds + (16 * t + r) * v_stride + 8 * g), pf, o[t]);
+      }
+    }
+  }
+
+  // ---- the row's sum over its four lanes; then the sink and the division, or the partial for the merge ----
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (!row_ok) return;
+  const float mn = m * scale;                                  // the maximum in the exponent's own unit
+  if (n_splits > 1) {
+    // (splits are for sequences of one token: the partial's row is the sequence's place in the launch and the head)
+    float* w = ws + (((size_t)blockIdx.y * nh + head) * n_splits + blockIdx.z) * (rank + 2);
+    if (g == 0) {
+      w[0] = mn;
+      w[1] = l;
+    }
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+      if (t < v_tiles)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int d = 16 * t + 4 * g + i;
+          if (d < rank) w[2 + d] = o[t][i];
+        }
+    return;
+  }
+  float a = 1.f;
+  if (sink) {
+    const float sk = sink[head];
+    const float top = fmaxf(mn, sk);
+    a = expf(mn - top);
+    l = l * a + expf(sk - top);
+  }
+  const float inv = a / l;
+  bf16* orow = out + ((size_t)(q0 + tq) * nh + head) * rank;
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+    if (t < v_tiles) {
+      const int d = 16 * t + 4 * g;
+      if (d + 4 <= rank) {
+        bf16x4 v = {(bf16)(o[t][0] * inv), (bf16)(o[t][1] * inv), (bf16)(o[t][2] * inv), (bf16)(o[t][3] * inv)};
+        *reinterpret_cast<bf16x4*>(orow + d) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (d + i < rank) orow[d + i] = (bf16)(o[t][i] * inv);
+      }
+    }
+}
+
+// out[row] = sum over the splits' partials, each scaled by exp(its maximum - the largest), then the sink.
+// One workgroup a row; the splits are added in order.
+__global__ __launch_bounds__(256) void latent_attn_merge_kernel(const float* __restrict__ ws, const float* __restrict__ sink,
+                                                               const int* __restrict__ seq_ids, const int* __restrict__ cu_q,
+                                                               bf16* __restrict__ out, int nh, int rank, int n_splits) {
+  const int row = blockIdx.x;                                  // (place in the launch) * heads + head
+  const int seq = seq_ids ? seq_ids[row / nh] : row / nh;
+  const size_t out_row = (size_t)cu_q[seq] * nh + row % nh;
+  const float* w = ws + (size_t)row * n_splits * (rank + 2);
+  float top = -INFINITY;
+  for (int z = 0; z < n_splits; ++z) top = fmaxf(top, w[(size_t)z * (rank + 2)]);
+  const float sk = sink ? sink[row % nh] : -INFINITY;
+  top = fmaxf(top, sk);
+  float l = sink ? expf(sk - top) : 0.f;
+  for (int z = 0; z < n_splits; ++z) {
+    const float mz = w[(size_t)z * (rank + 2)];
+    if (mz != -INFINITY) l += w[(size_t)z * (rank + 2) + 1] * expf(mz - top);
+  }
+  const float inv = 1.f / l;
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    float acc = 0.f;
+    for (int z = 0; z < n_splits; ++z) {
+      const float mz = w[(size_t)z * (rank + 2)];
+      if (mz != -INFINITY) acc += w[(size_t)z * (rank + 2) + 2 + d] * expf(mz - top);
+    }
+    out[out_row * rank + d] = (bf16)(acc * inv);
+  }
+}
+
+template <int RT, int QS>
+static int launch_latent_mfma(hipStream_t st, dim3 grid, size_t lds, const bf16* q, const bf16* cache, const float* sink,
+                              const int* block_table, int table_stride, const int* seq_ids, const int* cu_q,
+                              const int* context_lens, bf16* out, float* ws, int nh, int rank, int rot, int page_size,
+                              int window, float scale, int split_keys, int n_splits) {
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<RT, QS>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return pa::fail("latent_attn_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<RT, QS>), grid, dim3(256), lds, st, q, cache, sink, block_table, table_stride,
+                     seq_ids, cu_q, context_lens, out, ws, nh, rank, rot, page_size, window, scale, split_keys, n_splits);
+  return 0;
+}
+
+static size_t latent_mfma_lds(int rank, int rot) {
+  const int dk_steps = (rank + rot + 31) / 32, v_tiles = (rank + 15) / 16;
+  return (size_t)(kLmKeys * (dk_steps * 32 + kLmPad) + v_tiles * 16 * (kLmKeys + kLmPad)) * sizeof(bf16);
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+// Sizes the matrix-core kernel takes: 16-byte rows, at most 512 + 64 elements.
+extern "C" int pa_latent_attn_mfma_supports(int rank, int rot, int page_size) {
+  return rank > 0 && rot >= 0 && rank % 8 == 0 && rot % 8 == 0 && rank <= 512 && rot <= 64 && page_size > 0 &&
+         latent_mfma_lds(rank, rot) <= 160 * 1024;
+}
+
+// 32-bit words of workspace for `n_seqs` sequences of one token in `n_splits` splits
+extern "C" long pa_latent_attn_mfma_workspace(int n_seqs, int nh, int rank, int n_splits) {
+  return n_splits > 1 ? (long)n_seqs * nh * n_splits * (rank + 2) : 0;
+}
+
+// q [tokens, heads, rank + rot] -> out [tokens, heads, rank] for the sequences seq_ids[0..n_seqs) (null: sequences
+// 0..n_seqs), each with cu_q[s+1] - cu_q[s] tokens ending at context_lens[s]; max_q_len bounds their tokens.
+// n_splits > 1 (sequences of one token only): the keys in splits of split_keys, partials in ws, merged here.
+extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cache, const float* sink, const int* block_table,
+                                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                                   void* ws, int n_seqs, int max_q_len, int nh, int rank, int rot, int page_size,
+                                   int window, float scale, int split_keys, int n_splits) {
+  if (n_seqs == 0) return 0;
+  PA_REQUIRE(pa_latent_attn_mfma_supports(rank, rot, page_size), "latent_attn_mfma: a latent of %d + %d is not a size it takes", rank, rot);
+  PA_REQUIRE(n_seqs > 0 && max_q_len > 0 && nh > 0 && table_stride > 0 && window >= 0,
+             "latent_attn_mfma: bad sizes seqs=%d q=%d heads=%d stride=%d window=%d", n_seqs, max_q_len, nh, table_stride, window);
+  PA_REQUIRE(scale > 0.f, "latent_attn_mfma: a scale of %g is not positive", (double)scale);
+  PA_REQUIRE(n_splits >= 1 && (n_splits == 1 || (split_keys > 0 && split_keys % kLmKeys == 0 && ws && max_q_len == 1)),
+             "latent_attn_mfma: %d splits of %d keys need a workspace, whole blocks and sequences of one token", n_splits, split_keys);
+  const long tiles = ((long)max_q_len * nh + kLmRows - 1) / kLmRows;
+  PA_REQUIRE(tiles <= 0x7fffffffL && n_seqs <= 65535 && n_splits <= 65535, "latent_attn_mfma: the grid %ld x %d x %d is too large", tiles, n_seqs, n_splits);
+  dim3 grid((unsigned)tiles, n_seqs, n_splits);
+  const size_t lds = latent_mfma_lds(rank, rot);
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+#define PA_LM(RT, QS)                                                                                                  \
+  rc = launch_latent_mfma<RT, QS>(st, grid, lds, (const bf16*)q, (const bf16*)cache, sink, block_table, table_stride,  \
+                                  seq_ids, cu_q, context_lens, (bf16*)out, (float*)ws, nh, rank, rot, page_size, window, \
+                                  scale, split_keys, n_splits)
+  if (rank <= 64) PA_LM(4, 4);
+  else if (rank <= 128) PA_LM(8, 6);
+  else if (rank <= 256) PA_LM(16, 10);
+  else PA_LM(32, 18);
+#undef PA_LM
+  if (rc) return rc;
+  if (int e = check_launch("latent_attn_mfma")) return e;
+  if (n_splits > 1) {
+    hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(n_seqs * nh), dim3(rank >= 256 ? 256 : 64), 0, st, (const float*)ws, sink,
+                       seq_ids, cu_q, (bf16*)out, nh, rank, n_splits);
+    return check_launch("latent_attn_merge");
+  }
+  return 0;
+}

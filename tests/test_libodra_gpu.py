@@ -184,6 +184,46 @@ def test_latent_attention_over_pages(gpu, dtype, H, rank, rot, page):
     assert float((no_sink - want[37:]).abs().max()) > 0.05
 
 
+@pytest.mark.parametrize("H,rank,rot,page", [(3, 48, 16, 4), (8, 128, 32, 16), (5, 72, 8, 8), (16, 512, 64, 16), (40, 256, 64, 32)])
+def test_latent_attention_on_the_matrix_cores(gpu, H, rank, rot, page):
+    """The bfloat16 kernel: portions of unequal length (one starting at position 0, one deep in its context, with a
+    far key made to stand out), then every sequence feeding one token with its keys in splits."""
+    from prelude_amd.ops import kernels as K
+    assert K.latent_attention_mfma_supported(rank, rot, page)
+    dtype, width, scale = "bfloat16", rank + rot, 0.09
+    ctx = [700, 45, 300, 1]
+    qn = [70, 45, 2, 1]
+    lat = [rnd((n, width), 60 + i, dtype) for i, n in enumerate(ctx)]
+    qs = [rnd((n, H, width), 70 + i, dtype) for i, n in enumerate(qn)]
+    qs[0][-1] = (lat[0][9].float() * 3.0).to(torch.bfloat16)[None, :].expand(H, width)
+    sink = torch.linspace(-3.0, 2.0, H)
+    cache, table = _paged(lat, page, gpu, dtype, seed=5)
+    cu = torch.tensor([0] + list(np.cumsum(qn)), dtype=torch.int32, device=gpu)
+    cl = torch.tensor(ctx, dtype=torch.int32, device=gpu)
+    q = torch.cat(qs).to(gpu)
+    for window in (0, 40):
+        out = torch.zeros((q.shape[0], H, rank), dtype=torch.bfloat16, device=gpu)
+        K.latent_attention_mfma(q, cache, sink.to(gpu), table, None, 4, cu, cl, out, max(qn), rank, window, scale)
+        want = torch.cat([_plain_latent_attention(qs[i], lat[i], sink, rank, scale, torch.arange(ctx[i] - qn[i], ctx[i]), window)
+                          for i in range(4)])
+        close(out, want, dtype, f"portions, window {window}", scale=1.0)
+    # a chosen list of sequences leaves the other rows alone
+    out = torch.zeros((q.shape[0], H, rank), dtype=torch.bfloat16, device=gpu)
+    K.latent_attention_mfma(q, cache, sink.to(gpu), table, torch.tensor([2, 0], dtype=torch.int32, device=gpu), 2, cu, cl, out,
+                            70, rank, 0, scale)
+    assert float(out[70:115].abs().max()) == 0.0 and float(out[:70].abs().max()) > 0
+    # single tokens, keys in splits (and one context within a single split)
+    ql = [rnd((1, H, width), 80 + i, dtype) for i in range(4)]
+    ql[0][0] = (lat[0][300].float() * 3.0).to(torch.bfloat16)[None, :].expand(H, width)
+    cu1 = torch.arange(5, dtype=torch.int32, device=gpu)
+    out = torch.zeros((4, H, rank), dtype=torch.bfloat16, device=gpu)
+    for window in (0, 290):
+        K.latent_attention_mfma(torch.cat(ql).to(gpu), cache, sink.to(gpu), table, None, 4, cu1, cl, out, 1, rank, window, scale,
+                                max_context=768)
+        want = torch.cat([_plain_latent_attention(ql[i], lat[i], sink, rank, scale, torch.tensor([ctx[i] - 1]), window) for i in range(4)])
+        close(out, want, dtype, f"single tokens in splits, window {window}", scale=1.0)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_keys_at_page_borders_and_first_tokens(gpu, dtype):
     """Every query position of a sequence from 0 on, one launch a token, against the whole: position p sees keys 0..p,
