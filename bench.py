@@ -52,6 +52,43 @@ QWEN3_06B = dict(QWEN3_4B, hidden_size=1024, intermediate_size=3072, num_hidden_
 SHAPES = {"0.6b": QWEN3_06B, "4b": QWEN3_4B, "8b": QWEN3_8B, "32b": QWEN3_32B}
 
 
+def _vocab(raw):
+    return raw["vocab_size"] if "vocab_size" in raw else raw["vocab"]
+
+
+# ``--arch libodra``: a decoder of the Libodra design (attention through a latent with a sink; dense and
+# table-routed expert feed-forwards) at layer sizes of a real model of that kind, beside a Qwen3 decoder of the
+# same width, depth, vocabulary and about the same weights read per token
+def libodra_shape(layers=12, width=2048, vocab=65536):
+    mixer = dict(heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, rot=dict(base=10000.0, dims=64),
+                 scale=192 ** -0.5)
+    dense = dict(kind="dense", ff=8192, limit=7.0)
+    moe = dict(kind="moe", expert=dict(ff=1408), router=dict(experts=64, top=6), shared=dict(ff=2816))
+    return dict(architecture="Libodra", vocab=vocab, width=width, norm=dict(eps=1e-6),
+                layers=[dict(type="latent_attention", mixer=mixer, mlp=dense if i % 3 == 0 else moe) for i in range(layers)])
+
+
+def qwen3_beside_libodra(layers=12, width=2048, vocab=65536):
+    return dict(QWEN3_4B, hidden_size=width, intermediate_size=8192, num_hidden_layers=layers, max_window_layers=layers,
+                num_attention_heads=16, num_key_value_heads=8, head_dim=128, vocab_size=vocab, tie_word_embeddings=False,
+                eos_token_id=1)
+
+
+def libodra_record(args):
+    """Prefill and decode throughput of the Libodra shape and of the Qwen3 shape beside it, same points."""
+    out = {"arch": "libodra", "dtype": args.dtype, "layers": args.layers or 12, "points": {}}
+    for name, raw in (("libodra", libodra_shape(args.layers or 12)), ("qwen3_beside", qwen3_beside_libodra(args.layers or 12))):
+        pts = {}
+        for t in (512, args.prefill_tokens):
+            sec = time_prefill(raw, args.dtype, t, reps=3)
+            pts[f"prefill_{t}"] = {"ms": round(sec * 1e3, 3), "tok_per_s": round(t / sec, 1)}
+        for b, ctx in ((1, args.context), (args.batch, args.context), (32, args.context)):
+            sec = decode_point(raw, args.dtype, b, ctx, max(8, args.steps // 2), max(2, args.warmup // 2), None)
+            pts[f"decode_b{b}_ctx{ctx}"] = {"ms": round(sec * 1e3, 3), "tok_per_s": round(b / sec, 1)}
+        out["points"][name] = pts
+    return out
+
+
 def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
     """The engine in its random-weights mode: the product's own loader, tensors drawn on the device."""
     from prelude_amd.config import EngineConfig
@@ -69,7 +106,7 @@ def release_memory():
 
 
 def weight_bytes(raw, el):
-    h, i, v = raw["hidden_size"], raw["intermediate_size"], raw["vocab_size"]
+    h, i, v = raw["hidden_size"], raw["intermediate_size"], _vocab(raw)
     nh, nkv, hd, L = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"], raw["num_hidden_layers"]
     per_layer = ((nh + 2 * nkv) * hd * h + nh * hd * h + 3 * i * h) * el + (2 * h + 2 * hd) * 4
     head = v * h * el           # the head matrix is read whole; the embedding (the same matrix when tied) only gathers rows
@@ -176,13 +213,13 @@ def decode_point(raw, dtype, batch, context, steps, warmup, layers_note, chunk=2
     total = steps + warmup
     eng = build_engine(raw, dtype, cache_tokens=batch * (context + 64), max_num_batched_tokens=max(8192, chunk))
     if churned:
-        ids = churned_requests(eng, batch, context - total, raw["vocab_size"], seed=batch)
-        sec = time_decode(eng, batch, steps, warmup, raw["vocab_size"], ids)
+        ids = churned_requests(eng, batch, context - total, _vocab(raw), seed=batch)
+        sec = time_decode(eng, batch, steps, warmup, _vocab(raw), ids)
         del eng
         release_memory()
         return sec
-    prefill_requests(eng, batch, context - total, chunk, raw["vocab_size"], seed=batch)
-    sec = time_decode(eng, batch, steps, warmup, raw["vocab_size"])
+    prefill_requests(eng, batch, context - total, chunk, _vocab(raw), seed=batch)
+    sec = time_decode(eng, batch, steps, warmup, _vocab(raw))
     del eng
     release_memory()
     return sec
@@ -197,7 +234,7 @@ def time_prefill(raw, dtype, tokens, reps):
     rng = np.random.default_rng(7)
     times = []
     for r in range(reps + 1):
-        p = rng.integers(0, raw["vocab_size"], size=tokens).tolist()
+        p = rng.integers(0, _vocab(raw), size=tokens).tolist()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         eng.step([StepEntry(100 + r, p, [tokens - 1])])
@@ -220,7 +257,7 @@ def time_mixed(raw, dtype, chunk, decoding, context, steps, warmup):
     from prelude_amd.engine import StepEntry
     total = steps + warmup
     rng = np.random.default_rng(11)
-    vocab = raw["vocab_size"]
+    vocab = _vocab(raw)
     lens = [int(x) for x in np.linspace(256, context - total - 1, decoding)]
     need = sum(-(-(n + total + 1) // 64) * 64 for n in lens) + total * (context + 64)
     eng = build_engine(raw, dtype, cache_tokens=need + 4096)
@@ -258,7 +295,7 @@ def time_requests(raw, dtype, requests, prompt_len, max_tokens, concurrency, **c
                        **cfg_overrides)
     llm = LLM.from_engine(eng)
     rng = np.random.default_rng(5)
-    prompts = [rng.integers(0, raw["vocab_size"] - 1000, size=prompt_len).tolist() for _ in range(requests)]
+    prompts = [rng.integers(0, _vocab(raw) - 1000, size=prompt_len).tolist() for _ in range(requests)]
     llm.generate(prompts[:min(concurrency, 8)], max_tokens=max_tokens, temperature=0.0)   # warm-up
     greedy = SamplingParams(temperature=0.0)
     session = llm.session()
@@ -287,6 +324,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 0.6B, 8B or 32B")
+    ap.add_argument("--arch", default="qwen3", choices=["qwen3", "libodra"],
+                    help="libodra: prefill and decode of the Libodra design at a real model's layer sizes beside a Qwen3 "
+                         "decoder of equal size, as one record (the default run and its record are Qwen3's)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the points at other batches and lengths")
     ap.add_argument("--no-prefill", action="store_true")
@@ -309,6 +349,9 @@ def main() -> int:
         return 2
 
     import torch
+    if args.arch == "libodra":
+        print(json.dumps(libodra_record(args)), flush=True)
+        return 0
     raw = dict(SHAPES[args.shape])
     name = f"Qwen3-{args.shape.upper()} shape"
     full_layers = raw["num_hidden_layers"]

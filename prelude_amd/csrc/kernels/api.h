@@ -205,6 +205,12 @@ int pa_moe_linear(void* stream, int x_dtype, int w_dtype, int y_dtype, const voi
                   int act);
 int pa_moe_combine(void* stream, int dtype, const float* y, const int* place, const float* weights, float weight,
                    const void* base, void* out, int tokens, int top, int width);
+// The same two products on the matrix cores (grouped_mfma.hip; bfloat16 operands, K a multiple of 8): the weight as
+// stored, [group, N, K].
+int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, const void* w, void* y, const int* offsets, const int* order,
+                       int entries, int experts, int top, int K, int N, int from_tokens, int act);
+int pa_head_linear_mfma(void* stream, const void* x, const void* w, void* y, int tokens, int heads, int K, int N, long xs_t,
+                        long xs_h, long ys_t, long ys_h);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,159 @@
+// Products with a weight per group of rows, on the matrix cores (bfloat16, 32-bit sums): the experts' products
+// (group = expert, rows = the step's entries in expert order) and the per-head maps of attention through a latent
+// (group = head, rows = tokens).
+//
+// y[row, n] = sum_k x[row, k] * w[group, n, k], the weight as stored ([out, in], in fastest).  A workgroup of four
+// wavefronts owns up to 64 rows of one group and 128 outputs: each wavefront two tiles of 16 outputs against the
+// four tiles of 16 rows, W^T tile as A (row = output), X^T as B (column = row of x), both straight from memory in
+// 16-byte pieces (v_mfma_f32_16x16x32_bf16: A row r, columns 8g..8g+7; B column r, rows 8g..8g+7; C column r,
+// rows 4g..4g+3).  A weight element is read once per 64 rows, and sums run over k in ascending steps of 32
+// whatever else the launch holds.
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+constexpr int kGmRows = 64;
+constexpr int kGmCols = 128;
+
+// xrow(m) / yrow(m): element offsets of row m's input and output, < 0 for a row that does not exist.
+template <typename TY, typename RowX, typename RowY>
+__device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const bf16* __restrict__ w, TY* __restrict__ y,
+                                             int K, int N, int n_rows, int n0, int act, RowX xrow, RowY yrow) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int row_tiles = (n_rows + 15) / 16;
+  long xo[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) xo[mt] = (mt * 16 + r < n_rows) ? xrow(mt * 16 + r) : -1;
+  const int nb = n0 + wave * 32;
+  const bf16* wr[2];
+  bool wok[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = nb + 16 * j + r;
+    wok[j] = n < N;
+    wr[j] = w + (size_t)(wok[j] ? n : 0) * K + 8 * g;
+  }
+  if (nb >= N) return;
+  f32x4 acc[2][4];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[j][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool kok = k0 + 8 * g + 8 <= K;
+    bf16x8 wf[2], xf[4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      wf[j] = bf16x8{};
+      if (kok && wok[j]) wf[j] = *reinterpret_cast<const bf16x8*>(wr[j] + k0);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      xf[mt] = bf16x8{};
+      if (mt < row_tiles && kok && xo[mt] >= 0) xf[mt] = *reinterpret_cast<const bf16x8*>(x + xo[mt] + k0 + 8 * g);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      if (mt < row_tiles) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[mt], acc[j][mt], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    if (mt * 16 + r >= n_rows) continue;
+    const long yo = yrow(mt * 16 + r);
+    if (yo < 0) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = nb + 16 * j + 4 * g + i;
+        if (n < N) {
+          float v = acc[j][mt][i];
+          if (act == 1) {
+            v = fmaxf(v, 0.f);
+            v = v * v;
+          }
+          y[yo + n] = from_f32<TY>(v);
+        }
+      }
+  }
+}
+
+// Experts: blockIdx.x walks the tiles of 64 positions of all experts in order (an expert with c entries has
+// ceil(c / 64) tiles; blocks beyond the last leave).  `from_tokens`: position p reads row order[p] / top of x.
+template <typename TY>
+__global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
+                                                             TY* __restrict__ y, const int* __restrict__ offsets,
+                                                             const int* __restrict__ order, int experts, int top, int K,
+                                                             int N, int from_tokens, int act) {
+  int tile = blockIdx.x, e = 0, p0 = 0, p1 = 0;
+  for (; e < experts; ++e) {
+    const int a = offsets[e], b = offsets[e + 1];
+    const int tiles = (b - a + kGmRows - 1) / kGmRows;
+    if (tile < tiles) {
+      p0 = a + tile * kGmRows;
+      p1 = p0 + kGmRows < b ? p0 + kGmRows : b;
+      break;
+    }
+    tile -= tiles;
+  }
+  if (e >= experts) return;
+  grouped_tile<TY>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, blockIdx.y * kGmCols, act,
+                   [&](int m) { return (long)(from_tokens ? order[p0 + m] / top : p0 + m) * K; },
+                   [&](int m) { return (long)(p0 + m) * N; });
+}
+
+// Heads: grid (tiles of 64 tokens, heads, chunks of 128 outputs).
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
+                                                              bf16* __restrict__ y, int tokens, int K, int N, long xs_t,
+                                                              long xs_h, long ys_t, long ys_h) {
+  const int t0 = blockIdx.x * kGmRows, h = blockIdx.y;
+  const int n_rows = tokens - t0 < kGmRows ? tokens - t0 : kGmRows;
+  grouped_tile<bf16>(x, w + (size_t)h * N * K, y, K, N, n_rows, blockIdx.z * kGmCols, 0,
+                     [&](int m) { return (long)(t0 + m) * xs_t + (long)h * xs_h; },
+                     [&](int m) { return (long)(t0 + m) * ys_t + (long)h * ys_h; });
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+// x [rows, K] bfloat16 (a row per token when from_tokens, else per position), w [experts, N, K] bfloat16,
+// y [entries, N] of y_dtype; K a multiple of 8.
+extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, const void* w, void* y, const int* offsets,
+                                  const int* order, int entries, int experts, int top, int K, int N, int from_tokens, int act) {
+  if (entries == 0) return 0;
+  PA_REQUIRE(entries > 0 && experts > 0 && top > 0 && K > 0 && N > 0 && K % 8 == 0, "moe_linear_mfma: bad sizes entries=%d experts=%d k=%d n=%d",
+             entries, experts, K, N);
+  PA_REQUIRE(act == 0 || act == 1, "moe_linear_mfma: unknown activation code %d", act);
+  dim3 grid((entries + kGmRows - 1) / kGmRows + experts, (N + kGmCols - 1) / kGmCols);
+  hipStream_t st = (hipStream_t)stream;
+  if (y_dtype == kBF16)
+    hipLaunchKernelGGL(moe_linear_mfma_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (bf16*)y, offsets, order,
+                       experts, top, K, N, from_tokens, act);
+  else if (y_dtype == kF32)
+    hipLaunchKernelGGL(moe_linear_mfma_kernel<float>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (float*)y, offsets, order,
+                       experts, top, K, N, from_tokens, act);
+  else
+    return pa::fail("moe_linear_mfma: unknown output type code %d", y_dtype);
+  return check_launch("moe_linear_mfma");
+}
+
+// y[t, h, n] = sum_k x[t, h, k] w[h, n, k]; strides in elements, multiples of 8 (16-byte pieces), K a multiple of 8.
+extern "C" int pa_head_linear_mfma(void* stream, const void* x, const void* w, void* y, int tokens, int heads, int K, int N,
+                                   long xs_t, long xs_h, long ys_t, long ys_h) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && heads > 0 && K > 0 && N > 0 && K % 8 == 0 && xs_t % 8 == 0 && xs_h % 8 == 0,
+             "head_linear_mfma: bad sizes tokens=%d heads=%d k=%d n=%d strides %ld %ld", tokens, heads, K, N, xs_t, xs_h);
+  PA_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0, "head_linear_mfma: operands are not 16-byte aligned");
+  PA_REQUIRE(heads <= 65535 && (N + kGmCols - 1) / kGmCols <= 65535, "head_linear_mfma: %d heads or %d outputs exceed the grid", heads, N);
+  dim3 grid((tokens + kGmRows - 1) / kGmRows, heads, (N + kGmCols - 1) / kGmCols);
+  hipLaunchKernelGGL(head_linear_mfma_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, (const bf16*)w, (bf16*)y, tokens,
+                     K, N, xs_t, xs_h, ys_t, ys_h);
+  return check_launch("head_linear_mfma");
+}

@@ -1127,17 +1127,42 @@ def rotate_pairs(x: torch.Tensor, out: torch.Tensor, inv_freq: Optional[torch.Te
                                     x.shape[1], x.shape[2], int(in_off), out.shape[2], int(out_off), int(width), int(rot_dims)))
 
 
-def head_linear(x: torch.Tensor, wt: torch.Tensor, out: torch.Tensor, k: int, n: int, x_off: int = 0, out_off: int = 0) -> None:
-    """out[t, h, out_off : out_off + n] = W[h] x[t, h, x_off : x_off + k] for x [T, heads, a], out [T, heads, b] and the
-    weight as ``wt`` [heads, k, n] (the transposes of the heads' matrices)."""
+class GroupedWeight:
+    """A weight per group (expert, head), [groups, out, in], as the grouped products read it: for bfloat16 with rows
+    of whole 16-byte pieces as it stands (``nk``: the matrix cores take it so), else transposed to [groups, in, out]
+    (``kn``: the vector-ALU product reads its column beside its neighbours')."""
+
+    def __init__(self, w: torch.Tensor):
+        if w.dim() != 3:
+            raise NativeError(f"grouped weight {tuple(w.shape)} is not [groups, out, in]")
+        self.groups, self.n, self.k = (int(d) for d in w.shape)
+        self.dtype, self.device = w.dtype, w.device
+        self.nk = self.kn = None
+        if w.dtype == torch.bfloat16 and self.k % 8 == 0:
+            self.nk = w.contiguous()
+        else:
+            self.kn = w.transpose(1, 2).contiguous()
+
+
+def head_linear(x: torch.Tensor, w: GroupedWeight, out: torch.Tensor, x_off: int = 0, out_off: int = 0) -> None:
+    """out[t, h, out_off : out_off + n] = W[h] x[t, h, x_off : x_off + k] for x [T, heads, a], out [T, heads, b] and a
+    weight per head ``w`` [heads, n, k]."""
+    k, n = w.k, w.n
+    wt = w.nk if w.nk is not None else w.kn
     _dev(x, wt, out)
-    if (x.dim() != 3 or out.dim() != 3 or x.shape[:2] != out.shape[:2] or tuple(wt.shape) != (x.shape[1], k, n)
-            or not (x.dtype == wt.dtype == out.dtype) or x_off + k > x.shape[2] or out_off + n > out.shape[2]):
-        raise NativeError(f"head_linear: x {tuple(x.shape)} / wt {tuple(wt.shape)} / out {tuple(out.shape)}")
+    if (x.dim() != 3 or out.dim() != 3 or x.shape[:2] != out.shape[:2] or w.groups != x.shape[1]
+            or not (x.dtype == w.dtype == out.dtype) or x_off + k > x.shape[2] or out_off + n > out.shape[2]):
+        raise NativeError(f"head_linear: x {tuple(x.shape)} / w [{w.groups}, {n}, {k}] / out {tuple(out.shape)}")
     el = x.element_size()
-    check(kernels().pa_head_linear(_stream(), _code(x), x.data_ptr() + x_off * el, _ptr(wt), out.data_ptr() + out_off * el,
-                                   x.shape[0], x.shape[1], int(k), int(n), x.shape[1] * x.shape[2], x.shape[2],
-                                   out.shape[1] * out.shape[2], out.shape[2]))
+    strides = (x.shape[1] * x.shape[2], x.shape[2], out.shape[1] * out.shape[2], out.shape[2])
+    if w.nk is not None and x.shape[2] % 8 == 0 and x_off % 8 == 0:
+        check(kernels().pa_head_linear_mfma(_stream(), x.data_ptr() + x_off * el, _ptr(wt), out.data_ptr() + out_off * el,
+                                            x.shape[0], x.shape[1], k, n, *strides))
+        return
+    if w.kn is None:
+        w.kn = w.nk.transpose(1, 2).contiguous()     # rows of x that are no whole 16-byte pieces: the other product, once
+    check(kernels().pa_head_linear(_stream(), _code(x), x.data_ptr() + x_off * el, _ptr(w.kn), out.data_ptr() + out_off * el,
+                                   x.shape[0], x.shape[1], k, n, *strides))
 
 
 def latent_attention_generic(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], block_table: torch.Tensor,
@@ -1199,20 +1224,24 @@ def moe_order(choice: torch.Tensor, experts: int, top: int) -> ExpertOrder:
     return ExpertOrder(offsets, order, place, n, int(experts), int(top))
 
 
-def moe_linear(x: torch.Tensor, wt: torch.Tensor, eo: ExpertOrder, from_tokens: bool, relu_squared_epilogue: bool = False,
+def moe_linear(x: torch.Tensor, w: GroupedWeight, eo: ExpertOrder, from_tokens: bool, relu_squared_epilogue: bool = False,
                out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """y[p] = act(W[expert of p] x[row of p]) over the ordered positions p; ``wt`` [E, k, n] (the experts' matrices
-    transposed); ``from_tokens``: x holds a row per token (position p reads its token's), else a row per position."""
+    """y[p] = act(W[expert of p] x[row of p]) over the ordered positions p; ``w`` [experts, n, k];
+    ``from_tokens``: x holds a row per token (position p reads its token's), else a row per position."""
+    wt = w.nk if w.nk is not None else w.kn
     _dev(x, wt)
-    e, k, n = wt.shape
+    k, n = w.k, w.n
     rows = eo.entries // eo.top if from_tokens else eo.entries
-    if x.dim() != 2 or tuple(x.shape) != (rows, k) or e != eo.experts or x.dtype != wt.dtype:
-        raise NativeError(f"moe_linear: x {tuple(x.shape)} {x.dtype} / wt {tuple(wt.shape)} {wt.dtype} for {eo.entries} entries")
+    if x.dim() != 2 or tuple(x.shape) != (rows, k) or w.groups != eo.experts or x.dtype != w.dtype:
+        raise NativeError(f"moe_linear: x {tuple(x.shape)} {x.dtype} / w [{w.groups}, {n}, {k}] {w.dtype} for {eo.entries} entries")
     out_dtype = out_dtype or x.dtype
     y = torch.empty((eo.entries, n), dtype=out_dtype, device=x.device)
-    check(kernels().pa_moe_linear(_stream(), _code(x), _code(wt), _CODES[out_dtype], _ptr(x), _ptr(wt), _ptr(y), _ptr(eo.offsets),
-                                  _ptr(eo.order), eo.entries, eo.experts, eo.top, k, n, 1 if from_tokens else 0,
-                                  1 if relu_squared_epilogue else 0))
+    args = (_ptr(x), _ptr(wt), _ptr(y), _ptr(eo.offsets), _ptr(eo.order), eo.entries, eo.experts, eo.top, k, n,
+            1 if from_tokens else 0, 1 if relu_squared_epilogue else 0)
+    if w.nk is not None:
+        check(kernels().pa_moe_linear_mfma(_stream(), _CODES[out_dtype], *args))
+    else:
+        check(kernels().pa_moe_linear(_stream(), _code(x), _code(wt), _CODES[out_dtype], *args))
     return y
 
 

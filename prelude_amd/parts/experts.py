@@ -47,9 +47,9 @@ class TableExperts(FeedForward):
     def load(self, tensors, dtype, device):
         n = self.num_experts
         self.table = tensors["table"]
-        # [expert, inner, outer] with the outer index fastest: what the experts' product reads
-        self.up_t = torch.stack([tensors[f"e{e}.up"].t() for e in range(n)]).contiguous()
-        self.down_t = torch.stack([tensors[f"e{e}.down"].t() for e in range(n)]).contiguous()
+        # one tensor [expert, out, in] per product
+        self.up_t = K.GroupedWeight(torch.stack([tensors[f"e{e}.up"] for e in range(n)]))
+        self.down_t = K.GroupedWeight(torch.stack([tensors[f"e{e}.down"] for e in range(n)]))
         if self.shared_size:
             self.shared_up = K.prepare_weight(tensors["shared.up"])
             self.shared_down = K.prepare_weight(tensors["shared.down"])

@@ -80,10 +80,10 @@ class LatentAttention(Mixer):
         self.w_down = K.prepare_weight(torch.cat([tensors["dq"], tensors["dkv"]], dim=0).contiguous())
         self.w_uq = K.prepare_weight(tensors["uq"])
         self.w_o = K.prepare_weight(tensors["o"])
-        # the per-head maps as [head, inner, outer], the outer index running fastest: W_uk[h] is [d, rank] as stored
-        # and is applied transposed (inner d), W_uv[h] is [v, rank] and is applied as it is (inner rank)
-        self.uk_t = tensors["uk"].reshape(nh, d, rank).contiguous()
-        self.uv_t = tensors["uv"].reshape(nh, v, rank).transpose(1, 2).contiguous()
+        # the per-head maps as [head, out, in]: W_uk[h] is [d, rank] as stored and is applied transposed (out rank,
+        # in d); W_uv[h] is [v, rank] and is applied as it is
+        self.uk_t = K.GroupedWeight(tensors["uk"].reshape(nh, d, rank).transpose(1, 2))
+        self.uv_t = K.GroupedWeight(tensors["uv"].reshape(nh, v, rank))
         self.q_norm, self.c_norm = tensors["dq.norm"], tensors["dkv.norm"]
         self.sinks = tensors["sink"] if self.sink else None
 
@@ -96,9 +96,9 @@ class LatentAttention(Mixer):
                            cache.latent if write_cache else None, self.q_rank, rank, r, self.rotary_dim, self.norm_eps)
         q = K.linear(cq, self.w_uq).view(-1, nh, d + r)
         ql = torch.empty((q.shape[0], nh, rank + r), dtype=q.dtype, device=q.device)
-        K.head_linear(q, self.uk_t, ql, d, rank)                                    # the key map, on the query side
+        K.head_linear(q, self.uk_t, ql)                                             # the key map, on the query side
         K.rotate_pairs(q, ql, freq, step.positions, d, rank, r, self.rotary_dim)
         ol = K.latent_attention(ql, cache.latent, self.sinks, g, step, rank, self.window, self.scale)
         o = torch.empty((q.shape[0], nh, v), dtype=q.dtype, device=q.device)
-        K.head_linear(ol, self.uv_t, o, rank, v)                                    # the value map, after the sum
+        K.head_linear(ol, self.uv_t, o)                                            # the value map, after the sum
         return K.linear(o.view(-1, nh * v), self.w_o, slices_ok=True)

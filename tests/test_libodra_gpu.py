@@ -111,16 +111,21 @@ def test_rotation_of_a_part_of_every_head(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,H,k,n", [(1, 3, 24, 48), (19, 5, 72, 16), (40, 2, 130, 300)])
+@pytest.mark.parametrize("T,H,k,n", [(1, 3, 24, 48), (19, 5, 72, 16), (40, 2, 130, 300), (150, 4, 128, 512)])
 def test_a_product_per_head(gpu, dtype, T, H, k, n):
     from prelude_amd.ops import kernels as K
     x = rnd((T, H, k + 5), 9, dtype)
     w = rnd((H, n, k), 10, dtype, 1 / math.sqrt(k))           # [head, out, in]
     out = torch.zeros((T, H, n + 3), dtype=TD[dtype], device=gpu)
-    K.head_linear(x.to(gpu), w.transpose(1, 2).contiguous().to(gpu), out, k, n, x_off=5, out_off=3)
+    K.head_linear(x.to(gpu), K.GroupedWeight(w.to(gpu)), out, x_off=5, out_off=3)
     want = torch.einsum("thk,hnk->thn", x.double()[..., 5:], w.double())
     close(out[..., 3:], want, dtype, "per-head product")
     assert float(out[..., :3].abs().max()) == 0.0
+    if k % 8 == 0:       # rows of whole 16-byte pieces: in bfloat16 the matrix cores take it
+        x8 = rnd((T, H, k + 8), 11, dtype)
+        out = torch.zeros((T, H, n + 3), dtype=TD[dtype], device=gpu)
+        K.head_linear(x8.to(gpu), K.GroupedWeight(w.to(gpu)), out, x_off=8, out_off=3)
+        close(out[..., 3:], torch.einsum("thk,hnk->thn", x8.double()[..., 8:], w.double()), dtype, "per-head product, aligned")
 
 
 def _paged(latents, page, gpu, dtype, seed=0):
@@ -243,10 +248,10 @@ def test_keys_at_page_borders_and_first_tokens(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("E,top,T", [(6, 2, 50), (5, 3, 1), (4, 1, 33), (9, 2, 300)])
-def test_experts_by_table(gpu, dtype, E, top, T):
+@pytest.mark.parametrize("E,top,T,ff", [(6, 2, 50, 24), (5, 3, 1, 24), (4, 1, 33, 20), (9, 2, 300, 136), (3, 2, 400, 24)])
+def test_experts_by_table(gpu, dtype, E, top, T, ff):
     from prelude_amd.ops import kernels as K
-    V, Wd, ff = 31, 80, 24
+    V, Wd = 31, 80
     g = torch.Generator().manual_seed(E * 100 + T)
     table = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(V)]).to(torch.int32)
     if top == 1:
@@ -265,8 +270,8 @@ def test_experts_by_table(gpu, dtype, E, top, T):
     for e in range(E):
         mine = order[offsets[e]:offsets[e + 1]]
         assert torch.equal(mine, torch.sort(mine).values), "and within an expert in their own order"
-    mid = K.moe_linear(x.to(gpu), up.transpose(1, 2).contiguous().to(gpu), eo, True, relu_squared_epilogue=True)
-    y = K.moe_linear(mid, down.transpose(1, 2).contiguous().to(gpu), eo, False, out_dtype=torch.float32)
+    mid = K.moe_linear(x.to(gpu), K.GroupedWeight(up.to(gpu)), eo, True, relu_squared_epilogue=True)
+    y = K.moe_linear(mid, K.GroupedWeight(down.to(gpu)), eo, False, out_dtype=torch.float32)
     out = K.moe_combine(y, eo, 1.0 / top, base.to(gpu), TD[dtype])
     want = base.double().clone()
     for t in range(T):
