@@ -72,13 +72,13 @@ _KERNEL_API = {
     "pa_rmsnorm_wide": (I, [P, I, P, P, I, c_long, P, P, P, P, I, I, F]),
     "pa_clamped_gate": (I, [P, I, P, P, I, I, F, F]),
     "pa_relu_squared": (I, [P, I, P, P, c_long]),
-    "pa_latent_prep": (I, [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, F]),
+    "pa_latent_prep": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F]),
     "pa_rotate_pairs": (I, [P, I, P, P, P, P, I, I, I, I, I, I, I, I]),
     "pa_head_linear": (I, [P, I, P, P, P, I, I, I, I, c_long, c_long, c_long, c_long]),
     "pa_latent_attn": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
     "pa_latent_attn_mfma_supports": (I, [I, I, I]),
     "pa_latent_attn_mfma_workspace": (c_long, [I, I, I, I]),
-    "pa_latent_attn_mfma": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I]),
+    "pa_latent_attn_mfma": (I, [P, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I]),
     "pa_moe_choices_by_table": (I, [P, P, P, P, I, I, I, I]),
     "pa_moe_order": (I, [P, P, I, I, P, P, P, P]),
     "pa_moe_linear": (I, [P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I]),

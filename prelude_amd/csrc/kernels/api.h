@@ -171,10 +171,11 @@ int pa_relu_squared(void* stream, int dtype, const void* x, void* out, long tota
 // ---- attention through a latent (latent.hip) ----
 // in [tokens, q_rank + rank + rot]: cq_out [tokens, q_rank] = RMSNorm(first part) * wq; into the cache row slots[t]
 // ([rank + rot] elements a token): RMSNorm(second part) * wc, then the third part with its first rot_dims elements
-// rotated in pairs (2i, 2i+1) by the angle position * inv_freq[i].  slots null: nothing is cached.
+// rotated in pairs (2i, 2i+1) by the angle position * inv_freq[i].  slots null: nothing is cached.  cache_t (or null):
+// [pages, rank, page_size], the normed latent once more with the token's offset in its page running fastest.
 int pa_latent_prep(void* stream, int dtype, const void* in, const float* wq, const float* wc, const float* inv_freq,
-                   const int* positions, const int* slots, void* cq_out, void* cache, int tokens, int q_rank, int rank,
-                   int rot, int rot_dims, float eps);
+                   const int* positions, const int* slots, void* cq_out, void* cache, void* cache_t, int page_size,
+                   int tokens, int q_rank, int rank, int rot, int rot_dims, float eps);
 // in [tokens, heads, in_stride] -> out [tokens, heads, out_stride]: `width` elements from in_off to out_off of every
 // head, the first rot_dims of them rotated in pairs
 int pa_rotate_pairs(void* stream, int dtype, const void* in, void* out, const float* inv_freq, const int* positions,
@@ -191,7 +192,7 @@ int pa_latent_attn(void* stream, int dtype, const void* q, const void* cache, co
 // token: keys in splits of split_keys, partials in ws (pa_latent_attn_mfma_workspace 32-bit words), merged in split order.
 int pa_latent_attn_mfma_supports(int rank, int rot, int page_size);
 long pa_latent_attn_mfma_workspace(int n_seqs, int nh, int rank, int n_splits);
-int pa_latent_attn_mfma(void* stream, const void* q, const void* cache, const float* sink, const int* block_table,
+int pa_latent_attn_mfma(void* stream, const void* q, const void* cache, const void* cache_t, const float* sink, const int* block_table,
                         int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, void* ws,
                         int n_seqs, int max_q_len, int nh, int rank, int rot, int page_size, int window, float scale,
                         int split_keys, int n_splits);

@@ -6,7 +6,8 @@
 // All heads read the same keys: one "KV head" of width rank + rot whose value is its own first `rank` elements.
 //
 //   pa_latent_prep    the merged down projection's row [q_rank | rank | rot]: RMS norm of the query latent (out),
-//                     RMS norm of c and rotation of the shared key part (into the paged cache)
+//                     RMS norm of c and rotation of the shared key part (into the paged cache; c a second time
+//                     transposed, where the cache keeps that copy for the matrix-core kernel)
 //   pa_rotate_pairs   rotation of a part of every head's vector by position, pairs (2i, 2i+1)
 //   pa_head_linear    y[t, h, :] = W[h] x[t, h, :], a product per head
 //   pa_latent_attn    causal softmax attention over the latent cache with a learned sink per head in the
@@ -29,7 +30,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ in, const float* __restrict__ wq,
                                                          const float* __restrict__ wc, const float* __restrict__ inv_freq,
                                                          const int* __restrict__ positions, const int* __restrict__ slots,
-                                                         T* __restrict__ cq_out, T* __restrict__ cache, int q_rank,
+                                                         T* __restrict__ cq_out, T* __restrict__ cache,
+                                                         T* __restrict__ cache_t, int page_size, int q_rank,
                                                          int rank, int rot, int rot_dims, float eps) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
@@ -56,7 +58,13 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ 
   if (slot < 0) return;
   T* dst = cache + (size_t)slot * (rank + rot);
   const float inv = rsqrtf(sc / (float)rank + eps);
-  for (int i = threadIdx.x; i < rank; i += blockDim.x) dst[i] = from_f32<T>(to_f32(row[q_rank + i]) * inv * wc[i]);
+  // the latent a second time, transposed ([page, element, offset]): the weighted sum's operand for the matrix cores
+  T* dst_t = cache_t ? cache_t + (size_t)(slot / page_size) * rank * page_size + slot % page_size : nullptr;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const T v = from_f32<T>(to_f32(row[q_rank + i]) * inv * wc[i]);
+    dst[i] = v;
+    if (dst_t) dst_t[(size_t)i * page_size] = v;
+  }
   const float p = (float)positions[t];
   const T* kr = row + q_rank + rank;
   for (int i = threadIdx.x; i < rot_dims / 2; i += blockDim.x) {
@@ -249,15 +257,17 @@ using namespace pa;
 
 extern "C" int pa_latent_prep(void* stream, int dtype, const void* in, const float* wq, const float* wc,
                               const float* inv_freq, const int* positions, const int* slots, void* cq_out, void* cache,
-                              int tokens, int q_rank, int rank, int rot, int rot_dims, float eps) {
+                              void* cache_t, int page_size, int tokens, int q_rank, int rank, int rot, int rot_dims, float eps) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && q_rank > 0 && rank > 0 && rot >= 0, "latent_prep: bad sizes tokens=%d q_rank=%d rank=%d rot=%d",
              tokens, q_rank, rank, rot);
   PA_REQUIRE(rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0, "latent_prep: %d rotated of %d is not an even part", rot_dims, rot);
   PA_REQUIRE(!slots || cache, "latent_prep: slots without a cache");
+  PA_REQUIRE(!cache_t || page_size > 0, "latent_prep: a transposed copy needs the page size");
   PA_BY_TYPE(dtype, "latent_prep",
              hipLaunchKernelGGL(latent_prep_kernel<T>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, (const T*)in, wq, wc,
-                                inv_freq, positions, slots, (T*)cq_out, (T*)cache, q_rank, rank, rot, rot_dims, eps));
+                                inv_freq, positions, slots, (T*)cq_out, (T*)cache, (T*)cache_t, page_size, q_rank, rank, rot,
+                                rot_dims, eps));
   return check_launch("latent_prep");
 }
 

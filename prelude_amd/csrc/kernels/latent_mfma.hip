@@ -4,7 +4,8 @@
 // of four wavefronts owns 64 consecutive rows of one sequence's portion (row = token * heads + head), 16 a
 // wavefront, and walks the keys in blocks of 32.  A block is brought into LDS once per workgroup: the vectors as
 // they lie in the cache (rows of rank + rot elements, the score's operand), and the first `rank` elements of each
-// again transposed ([element][key]: the operand of the weighted sum, whose contraction runs over keys).
+// again transposed ([element][key]: the operand of the weighted sum, whose contraction runs over keys).  The cache
+// keeps that transposed copy itself ([pages, rank, page]), written once per token, so both are copied in 16-byte pieces.
 //
 //   S^T = K Q^T     A = 16 keys x 32 elements from LDS, B = the wavefront's queries, kept in registers
 //   O^T = V^T P^T   A = 16 elements x 32 keys from the transposed copy, B = the probabilities just computed
@@ -35,8 +36,8 @@ __device__ __forceinline__ f32x4 mfma16l(bf16x8 a, bf16x8 b, f32x4 c) {
 // registers (rank + rot <= 32 QS).
 template <int RT, int QS>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ cache, const float* __restrict__ sink,
-    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
+    const bf16* __restrict__ q, const bf16* __restrict__ cache, const bf16* __restrict__ cache_t,
+    const float* __restrict__ sink, const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
     float* __restrict__ ws, int nh, int rank, int rot, int page_size, int window, float scale, int split_keys,
     int n_splits) {
@@ -99,27 +100,60 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   float m = -INFINITY, l = 0.f;
   const float c = scale * kLog2eL;
   const int chunks = dk_steps * 4;                             // 16-byte pieces of a staged row
+  const bool wave_active = rb + wave * 16 < rows;              // a wavefront without rows of its own only helps staging
 
-  for (int b0 = lo_wg; b0 < end_wg; b0 += kLmKeys) {
-    __syncthreads();
-    // ---- stage the block: rows as they are, and their first `rank` elements transposed ----
-    // (neighbouring threads take neighbouring keys, so that the transposed 2-byte stores of a wavefront fall into
-    // one row of the copy instead of into rows a multiple of 32 banks apart)
-    for (int i = threadIdx.x; i < kLmKeys * chunks; i += 256) {
+  // A block's pieces, a thread's share held in registers between their loads and their stores into LDS, so that the
+  // loads of the next block are in flight while this block is worked on.  Rows: piece i is key i % 32, elements
+  // 8 (i / 32)...; the transposed copy: piece i is element i / 4, keys 8 (i % 4)... (pages hold multiples of 8 keys,
+  // so eight keys from a multiple of 8 lie in one page).
+  constexpr int KC = (kLmKeys * QS * 4 + 255) / 256;
+  constexpr int VC = (RT * 16 * 4 + 255) / 256;
+  bf16x8 kreg[KC], vreg[VC];
+  auto load_block = [&](int b0) {
+#pragma unroll
+    for (int cI = 0; cI < KC; ++cI) {
+      const int i = threadIdx.x + 256 * cI;
       const int key = i % kLmKeys, ch = i / kLmKeys;
       const int kidx = b0 + key;
       bf16x8 v = {};
-      if (kidx < end_wg && 8 * ch + 8 <= dk) {
+      if (ch < chunks && kidx < end_wg && 8 * ch + 8 <= dk) {
         const int page = table[kidx / page_size];
         if (page >= 0) v = *reinterpret_cast<const bf16x8*>(cache + ((size_t)page * page_size + kidx % page_size) * dk + 8 * ch);
       }
-      *reinterpret_cast<bf16x8*>(k_lds + key * k_stride + 8 * ch) = v;
-      if (8 * ch < v_tiles * 16) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v_lds[(8 * ch + j) * v_stride + key] = (8 * ch + j < rank) ? v[j] : (bf16)0.f;
-      }
+      kreg[cI] = v;
     }
+#pragma unroll
+    for (int cI = 0; cI < VC; ++cI) {
+      const int i = threadIdx.x + 256 * cI;
+      const int vrow = i / 4, kidx = b0 + 8 * (i % 4);
+      bf16x8 v = {};
+      if (vrow < rank && kidx < end_wg) {
+        const int page = table[kidx / page_size];
+        if (page >= 0) v = *reinterpret_cast<const bf16x8*>(cache_t + ((size_t)page * rank + vrow) * page_size + kidx % page_size);
+      }
+      vreg[cI] = v;
+    }
+  };
+  auto store_block = [&]() {
+#pragma unroll
+    for (int cI = 0; cI < KC; ++cI) {
+      const int i = threadIdx.x + 256 * cI;
+      if (i / kLmKeys < chunks) *reinterpret_cast<bf16x8*>(k_lds + (i % kLmKeys) * k_stride + 8 * (i / kLmKeys)) = kreg[cI];
+    }
+#pragma unroll
+    for (int cI = 0; cI < VC; ++cI) {
+      const int i = threadIdx.x + 256 * cI;
+      if (i / 4 < v_tiles * 16) *reinterpret_cast<bf16x8*>(v_lds + (i / 4) * v_stride + 8 * (i % 4)) = vreg[cI];
+    }
+  };
+
+  if (lo_wg < end_wg) load_block(lo_wg);
+  for (int b0 = lo_wg; b0 < end_wg; b0 += kLmKeys) {
     __syncthreads();
+    store_block();
+    __syncthreads();
+    if (b0 + kLmKeys < end_wg) load_block(b0 + kLmKeys);
+    if (!wave_active) continue;
     // ---- scores of 32 keys for this wavefront's 16 rows ----
     f32x4 s[2];
 #pragma unroll
@@ -245,7 +279,7 @@ __global__ __launch_bounds__(256) void latent_attn_merge_kernel(const float* __r
 }
 
 template <int RT, int QS>
-static int launch_latent_mfma(hipStream_t st, dim3 grid, size_t lds, const bf16* q, const bf16* cache, const float* sink,
+static int launch_latent_mfma(hipStream_t st, dim3 grid, size_t lds, const bf16* q, const bf16* cache, const bf16* cache_t, const float* sink,
                               const int* block_table, int table_stride, const int* seq_ids, const int* cu_q,
                               const int* context_lens, bf16* out, float* ws, int nh, int rank, int rot, int page_size,
                               int window, float scale, int split_keys, int n_splits) {
@@ -256,7 +290,7 @@ static int launch_latent_mfma(hipStream_t st, dim3 grid, size_t lds, const bf16*
     if (e != hipSuccess) return pa::fail("latent_attn_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
-  hipLaunchKernelGGL((latent_attn_mfma_kernel<RT, QS>), grid, dim3(256), lds, st, q, cache, sink, block_table, table_stride,
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<RT, QS>), grid, dim3(256), lds, st, q, cache, cache_t, sink, block_table, table_stride,
                      seq_ids, cu_q, context_lens, out, ws, nh, rank, rot, page_size, window, scale, split_keys, n_splits);
   return 0;
 }
@@ -270,9 +304,9 @@ static size_t latent_mfma_lds(int rank, int rot) {
 
 using namespace pa;
 
-// Sizes the matrix-core kernel takes: 16-byte rows, at most 512 + 64 elements.
+// Sizes the matrix-core kernel takes: 16-byte rows, at most 512 + 64 elements, pages of a multiple of 8 keys.
 extern "C" int pa_latent_attn_mfma_supports(int rank, int rot, int page_size) {
-  return rank > 0 && rot >= 0 && rank % 8 == 0 && rot % 8 == 0 && rank <= 512 && rot <= 64 && page_size > 0 &&
+  return rank > 0 && rot >= 0 && rank % 8 == 0 && rot % 8 == 0 && rank <= 512 && rot <= 64 && page_size > 0 && page_size % 8 == 0 &&
          latent_mfma_lds(rank, rot) <= 160 * 1024;
 }
 
@@ -281,10 +315,11 @@ extern "C" long pa_latent_attn_mfma_workspace(int n_seqs, int nh, int rank, int 
   return n_splits > 1 ? (long)n_seqs * nh * n_splits * (rank + 2) : 0;
 }
 
-// q [tokens, heads, rank + rot] -> out [tokens, heads, rank] for the sequences seq_ids[0..n_seqs) (null: sequences
+// q [tokens, heads, rank + rot], cache [pages, page, rank + rot] and its latents transposed, cache_t [pages, rank, page]
+// -> out [tokens, heads, rank] for the sequences seq_ids[0..n_seqs) (null: sequences
 // 0..n_seqs), each with cu_q[s+1] - cu_q[s] tokens ending at context_lens[s]; max_q_len bounds their tokens.
 // n_splits > 1 (sequences of one token only): the keys in splits of split_keys, partials in ws, merged here.
-extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cache, const float* sink, const int* block_table,
+extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cache, const void* cache_t, const float* sink, const int* block_table,
                                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                                    void* ws, int n_seqs, int max_q_len, int nh, int rank, int rot, int page_size,
                                    int window, float scale, int split_keys, int n_splits) {
@@ -292,6 +327,7 @@ extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cach
   PA_REQUIRE(pa_latent_attn_mfma_supports(rank, rot, page_size), "latent_attn_mfma: a latent of %d + %d is not a size it takes", rank, rot);
   PA_REQUIRE(n_seqs > 0 && max_q_len > 0 && nh > 0 && table_stride > 0 && window >= 0,
              "latent_attn_mfma: bad sizes seqs=%d q=%d heads=%d stride=%d window=%d", n_seqs, max_q_len, nh, table_stride, window);
+  PA_REQUIRE(cache && cache_t, "latent_attn_mfma: needs the cache and its transposed copy");
   PA_REQUIRE(scale > 0.f, "latent_attn_mfma: a scale of %g is not positive", (double)scale);
   PA_REQUIRE(n_splits >= 1 && (n_splits == 1 || (split_keys > 0 && split_keys % kLmKeys == 0 && ws && max_q_len == 1)),
              "latent_attn_mfma: %d splits of %d keys need a workspace, whole blocks and sequences of one token", n_splits, split_keys);
@@ -302,7 +338,7 @@ extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cach
   hipStream_t st = (hipStream_t)stream;
   int rc;
 #define PA_LM(RT, QS)                                                                                                  \
-  rc = launch_latent_mfma<RT, QS>(st, grid, lds, (const bf16*)q, (const bf16*)cache, sink, block_table, table_stride,  \
+  rc = launch_latent_mfma<RT, QS>(st, grid, lds, (const bf16*)q, (const bf16*)cache, (const bf16*)cache_t, sink, block_table, table_stride,  \
                                   seq_ids, cu_q, context_lens, (bf16*)out, (float*)ws, nh, rank, rot, page_size, window, \
                                   scale, split_keys, n_splits)
   if (rank <= 64) PA_LM(4, 4);

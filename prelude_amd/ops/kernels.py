@@ -1088,10 +1088,11 @@ def relu_squared(x: torch.Tensor) -> torch.Tensor:
 # Attention through a latent
 def latent_prep(down: torch.Tensor, q_weight: torch.Tensor, c_weight: torch.Tensor, inv_freq: Optional[torch.Tensor],
                 positions: torch.Tensor, slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], q_rank: int,
-                rank: int, rot: int, rot_dims: int, eps: float) -> torch.Tensor:
+                rank: int, rot: int, rot_dims: int, eps: float, cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The merged down projection [T, q_rank + rank + rot]: returns the normed query latent [T, q_rank]; writes the
-    normed latent and the rotated shared key part of every token into ``cache`` [pages, page, rank + rot] at ``slots``."""
-    _dev(down, q_weight, c_weight, inv_freq, positions, slots, cache)
+    normed latent and the rotated shared key part of every token into ``cache`` [pages, page, rank + rot] at ``slots``,
+    and the latent once more into ``cache_t`` [pages, rank, page] where the cache keeps that copy."""
+    _dev(down, q_weight, c_weight, inv_freq, positions, slots, cache, cache_t)
     _f32(q_weight, "query latent norm weight")
     _f32(c_weight, "latent norm weight")
     _f32(inv_freq, "rotary frequencies")
@@ -1105,9 +1106,13 @@ def latent_prep(down: torch.Tensor, q_weight: torch.Tensor, c_weight: torch.Tens
         _i32(slots, "slots")
         if slots.shape != (t,) or cache is None or cache.dim() != 3 or cache.shape[2] != rank + rot or cache.dtype != down.dtype:
             raise NativeError(f"latent_prep: cache must be [pages, page, {rank + rot}] of {down.dtype}")
+        if cache_t is not None and (cache_t.dtype != cache.dtype or tuple(cache_t.shape) != (cache.shape[0], rank, cache.shape[1])):
+            raise NativeError(f"latent_prep: the transposed copy must be [pages, {rank}, page] of {cache.dtype}")
     cq = torch.empty((t, q_rank), dtype=down.dtype, device=down.device)
+    caching = slots is not None
     check(kernels().pa_latent_prep(_stream(), _code(down), _ptr(down), _ptr(q_weight), _ptr(c_weight), _ptr(inv_freq),
-                                   _ptr(positions), _ptr(slots), _ptr(cq), _ptr(cache) if slots is not None else None, t,
+                                   _ptr(positions), _ptr(slots), _ptr(cq), _ptr(cache) if caching else None,
+                                   _ptr(cache_t) if caching else None, cache.shape[1] if caching else 0, t,
                                    q_rank, rank, rot, rot_dims, float(eps)))
     return cq
 
@@ -1272,16 +1277,18 @@ def latent_attention_mfma_supported(rank: int, rot: int, page_size: int) -> bool
     return bool(kernels().pa_latent_attn_mfma_supports(int(rank), int(rot), int(page_size)))
 
 
-def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], block_table: torch.Tensor,
+def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, cache_t: torch.Tensor, sink: Optional[torch.Tensor], block_table: torch.Tensor,
                           seq_ids: Optional[torch.Tensor], n_seqs: int, cu_q: torch.Tensor, context_lens: torch.Tensor,
                           out: torch.Tensor, max_q_len: int, rank: int, window: int, scale: float,
                           max_context: int = 0) -> None:
     """The matrix-core kernel for the sequences ``seq_ids`` (None: all ``n_seqs`` of the step); writes their rows of
     ``out`` [T, heads, rank].  ``max_context`` > 0 with ``max_q_len`` 1 cuts the keys into splits of
     ``LATENT_SPLIT_KEYS`` whose partials a second kernel merges: what fills the chip when every sequence feeds one token."""
-    _dev(q, cache, sink, block_table, seq_ids, cu_q, context_lens, out)
+    _dev(q, cache, cache_t, sink, block_table, seq_ids, cu_q, context_lens, out)
     _f32(sink, "sink")
     t, nh, dk = q.shape
+    if cache_t is None or cache_t.dtype != torch.bfloat16 or tuple(cache_t.shape) != (cache.shape[0], rank, cache.shape[1]):
+        raise NativeError(f"latent_attention_mfma: the transposed copy must be [pages, {rank}, page] of bfloat16")
     if q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16 or cache.dim() != 3 or cache.shape[2] != dk \
             or tuple(out.shape) != (t, nh, rank) or out.dtype != torch.bfloat16 or (sink is not None and sink.shape != (nh,)):
         raise NativeError(f"latent_attention_mfma: q {tuple(q.shape)} {q.dtype} / cache {tuple(cache.shape)} / out {tuple(out.shape)}")
@@ -1291,27 +1298,27 @@ def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, sink: Optional[t
     if max_q_len == 1 and max_context > LATENT_SPLIT_KEYS:
         splits = -(-int(max_context) // LATENT_SPLIT_KEYS)
         ws = torch.empty(int(kernels().pa_latent_attn_mfma_workspace(n_seqs, nh, rank, splits)), dtype=torch.float32, device=q.device)
-    check(kernels().pa_latent_attn_mfma(_stream(), _ptr(q), _ptr(cache), _ptr(sink), _ptr(block_table), block_table.shape[1],
+    check(kernels().pa_latent_attn_mfma(_stream(), _ptr(q), _ptr(cache), _ptr(cache_t), _ptr(sink), _ptr(block_table), block_table.shape[1],
                                         _ptr(seq_ids), _ptr(cu_q), _ptr(context_lens), _ptr(out), _ptr(ws), int(n_seqs),
                                         int(max_q_len), nh, int(rank), dk - int(rank), cache.shape[1], int(window), float(scale),
                                         LATENT_SPLIT_KEYS, splits))
 
 
 def latent_attention(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], group, step, rank: int,
-                     window: int, scale: float) -> torch.Tensor:
+                     window: int, scale: float, cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of one step over a cache of latents; picks the kernel for the sizes at hand (``group``: the
     step's ``GroupStep`` of the cache group, ``step``: the ``StepBatch``).  bfloat16 with sizes the matrix-core
     kernel takes: single tokens in splits of their keys, portions a launch of their own; everything else
     (float32, other sizes) the kernel on the vector ALU."""
-    if (q.dtype == torch.bfloat16 and step.decode_seqs is not None and scale > 0
+    if (q.dtype == torch.bfloat16 and cache_t is not None and step.decode_seqs is not None and scale > 0
             and latent_attention_mfma_supported(rank, q.shape[2] - rank, cache.shape[1])):
         out = torch.empty((q.shape[0], q.shape[1], rank), dtype=q.dtype, device=q.device)
         if step.n_decode:
             every = step.n_prefill == 0 and step.n_decode == step.num_seqs
-            latent_attention_mfma(q, cache, sink, group.block_table, None if every else step.decode_seqs, step.n_decode,
+            latent_attention_mfma(q, cache, cache_t, sink, group.block_table, None if every else step.decode_seqs, step.n_decode,
                                   step.cu_q, step.context_lens, out, 1, rank, window, scale, max_context=step.max_decode_context)
         if step.n_prefill:
-            latent_attention_mfma(q, cache, sink, group.block_table, step.prefill_seqs, step.n_prefill, step.cu_q,
+            latent_attention_mfma(q, cache, cache_t, sink, group.block_table, step.prefill_seqs, step.n_prefill, step.cu_q,
                                   step.context_lens, out, step.max_prefill_q, rank, window, scale)
         return out
     return latent_attention_generic(q, cache, sink, group.block_table, step.seq_of_token, step.positions, rank, window, scale)

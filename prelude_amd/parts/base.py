@@ -147,6 +147,7 @@ class LatentLayerCache:
     """What a mixer that attends through a latent gets: one vector a token, in pages."""
     latent: torch.Tensor   # [pages, page_size, rank + rot]
     group: int
+    latent_t: Optional[torch.Tensor] = None   # [pages, rank, page_size]: the latents once more, transposed
 
 
 @dataclasses.dataclass(frozen=True)
@@ -154,16 +155,25 @@ class LatentCacheSpec(PagedCacheSpec):
     """One vector per token, in pages: a latent of ``rank`` elements that stands for the keys and values of all
     heads, followed by ``rot`` elements of a rotated key part the heads share.  Layout per cache slot
     ``[pages, page_size, rank + rot]``: a token's vector is one run of memory, read whole for a score and by its
-    first ``rank`` elements as the value."""
+    first ``rank`` elements as the value.  In bfloat16 with pages of a multiple of 8 tokens the latent is kept a
+    second time with the tokens of a page running fastest (``[pages, rank, page_size]``): the weighted sum on the
+    matrix cores contracts over keys and loads eight of them in one piece from there."""
     rank: int
     rot: int
     window: int = 0
 
+    @staticmethod
+    def keeps_transposed(page_size: int, dtype: torch.dtype) -> bool:
+        return dtype == torch.bfloat16 and page_size % 8 == 0
+
     def bytes_per_token(self, element_size: int) -> int:
-        return (self.rank + self.rot) * element_size
+        # counted with the transposed copy, which serving (bfloat16, the usual page sizes) keeps
+        return (2 * self.rank + self.rot) * element_size
 
     def allocate(self, pages, page_size, dtype, device, group):
-        return LatentLayerCache(torch.zeros((pages, page_size, self.rank + self.rot), dtype=dtype, device=device), group)
+        t = torch.zeros((pages, self.rank, page_size), dtype=dtype, device=device) \
+            if self.keeps_transposed(page_size, dtype) else None
+        return LatentLayerCache(torch.zeros((pages, page_size, self.rank + self.rot), dtype=dtype, device=device), group, t)
 
 
 @dataclasses.dataclass(frozen=True)

@@ -93,12 +93,13 @@ class LatentAttention(Mixer):
         freq = self.rope.inv_freq if self.rope is not None else None
         down = K.linear(x, self.w_down)
         cq = K.latent_prep(down, self.q_norm, self.c_norm, freq, step.positions, g.slots if write_cache else None,
-                           cache.latent if write_cache else None, self.q_rank, rank, r, self.rotary_dim, self.norm_eps)
+                           cache.latent if write_cache else None, self.q_rank, rank, r, self.rotary_dim, self.norm_eps,
+                           cache_t=cache.latent_t if write_cache else None)
         q = K.linear(cq, self.w_uq).view(-1, nh, d + r)
         ql = torch.empty((q.shape[0], nh, rank + r), dtype=q.dtype, device=q.device)
         K.head_linear(q, self.uk_t, ql)                                             # the key map, on the query side
         K.rotate_pairs(q, ql, freq, step.positions, d, rank, r, self.rotary_dim)
-        ol = K.latent_attention(ql, cache.latent, self.sinks, g, step, rank, self.window, self.scale)
+        ol = K.latent_attention(ql, cache.latent, self.sinks, g, step, rank, self.window, self.scale, cache_t=cache.latent_t)
         o = torch.empty((q.shape[0], nh, v), dtype=q.dtype, device=q.device)
         K.head_linear(ol, self.uv_t, o)                                            # the value map, after the sum
         return K.linear(o.view(-1, nh * v), self.w_o, slices_ok=True)

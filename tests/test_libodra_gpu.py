@@ -82,8 +82,10 @@ def test_latent_prep_norms_rotates_and_caches(gpu, dtype, q_rank, rank, rot, dim
     slots = torch.randperm(page * pages)[:T].to(torch.int32)
     freq = torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=torch.float32) if dims else None
     cache = torch.zeros((pages, page, rank + rot), dtype=TD[dtype], device=gpu)
+    cache_t = torch.zeros((pages, rank, page), dtype=TD[dtype], device=gpu)
     cq = K.latent_prep(down.to(gpu), wq.to(gpu), wc.to(gpu), None if freq is None else freq.to(gpu), pos.to(gpu), slots.to(gpu),
-                       cache, q_rank, rank, rot, dims, eps)
+                       cache, q_rank, rank, rot, dims, eps, cache_t=cache_t)
+    assert torch.equal(cache_t.transpose(1, 2), cache[:, :, :rank]), "the transposed copy holds the same latents"
     d = down.double()
     close(cq, pl.unit_rms(d[:, :q_rank], eps) * wq.double(), dtype, "query latent")
     got = cache.reshape(-1, rank + rot)[slots.long().to(gpu)]
@@ -189,7 +191,7 @@ def test_latent_attention_over_pages(gpu, dtype, H, rank, rot, page):
     assert float((no_sink - want[37:]).abs().max()) > 0.05
 
 
-@pytest.mark.parametrize("H,rank,rot,page", [(3, 48, 16, 4), (8, 128, 32, 16), (5, 72, 8, 8), (16, 512, 64, 16), (40, 256, 64, 32)])
+@pytest.mark.parametrize("H,rank,rot,page", [(3, 48, 16, 8), (8, 128, 32, 16), (5, 72, 8, 8), (16, 512, 64, 16), (40, 256, 64, 32), (2, 64, 0, 24)])
 def test_latent_attention_on_the_matrix_cores(gpu, H, rank, rot, page):
     """The bfloat16 kernel: portions of unequal length (one starting at position 0, one deep in its context, with a
     far key made to stand out), then every sequence feeding one token with its keys in splits."""
@@ -203,18 +205,19 @@ def test_latent_attention_on_the_matrix_cores(gpu, H, rank, rot, page):
     qs[0][-1] = (lat[0][9].float() * 3.0).to(torch.bfloat16)[None, :].expand(H, width)
     sink = torch.linspace(-3.0, 2.0, H)
     cache, table = _paged(lat, page, gpu, dtype, seed=5)
+    cache_t = cache[:, :, :rank].transpose(1, 2).contiguous()          # [pages, rank, page]: the copy the cache keeps
     cu = torch.tensor([0] + list(np.cumsum(qn)), dtype=torch.int32, device=gpu)
     cl = torch.tensor(ctx, dtype=torch.int32, device=gpu)
     q = torch.cat(qs).to(gpu)
     for window in (0, 40):
         out = torch.zeros((q.shape[0], H, rank), dtype=torch.bfloat16, device=gpu)
-        K.latent_attention_mfma(q, cache, sink.to(gpu), table, None, 4, cu, cl, out, max(qn), rank, window, scale)
+        K.latent_attention_mfma(q, cache, cache_t, sink.to(gpu), table, None, 4, cu, cl, out, max(qn), rank, window, scale)
         want = torch.cat([_plain_latent_attention(qs[i], lat[i], sink, rank, scale, torch.arange(ctx[i] - qn[i], ctx[i]), window)
                           for i in range(4)])
         close(out, want, dtype, f"portions, window {window}", scale=1.0)
     # a chosen list of sequences leaves the other rows alone
     out = torch.zeros((q.shape[0], H, rank), dtype=torch.bfloat16, device=gpu)
-    K.latent_attention_mfma(q, cache, sink.to(gpu), table, torch.tensor([2, 0], dtype=torch.int32, device=gpu), 2, cu, cl, out,
+    K.latent_attention_mfma(q, cache, cache_t, sink.to(gpu), table, torch.tensor([2, 0], dtype=torch.int32, device=gpu), 2, cu, cl, out,
                             70, rank, 0, scale)
     assert float(out[70:115].abs().max()) == 0.0 and float(out[:70].abs().max()) > 0
     # single tokens, keys in splits (and one context within a single split)
@@ -223,7 +226,7 @@ def test_latent_attention_on_the_matrix_cores(gpu, H, rank, rot, page):
     cu1 = torch.arange(5, dtype=torch.int32, device=gpu)
     out = torch.zeros((4, H, rank), dtype=torch.bfloat16, device=gpu)
     for window in (0, 290):
-        K.latent_attention_mfma(torch.cat(ql).to(gpu), cache, sink.to(gpu), table, None, 4, cu1, cl, out, 1, rank, window, scale,
+        K.latent_attention_mfma(torch.cat(ql).to(gpu), cache, cache_t, sink.to(gpu), table, None, 4, cu1, cl, out, 1, rank, window, scale,
                                 max_context=768)
         want = torch.cat([_plain_latent_attention(ql[i], lat[i], sink, rank, scale, torch.tensor([ctx[i] - 1]), window) for i in range(4)])
         close(out, want, dtype, f"single tokens in splits, window {window}", scale=1.0)
