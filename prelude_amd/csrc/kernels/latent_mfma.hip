@@ -5,7 +5,8 @@
 // wavefront, and walks the keys in blocks of 32.  A block is brought into LDS once per workgroup: the vectors as
 // they lie in the cache (rows of rank + rot elements, the score's operand), and the first `rank` elements of each
 // again transposed ([element][key]: the operand of the weighted sum, whose contraction runs over keys).  The cache
-// keeps that transposed copy itself ([pages, rank, page]), written once per token, so both are copied in 16-byte pieces.
+// keeps that transposed copy itself ([pages, rank, page]), written once per token, so both are copied in 16-byte
+// pieces, from memory straight into LDS.
 //
 //   S^T = K Q^T     A = 16 keys x 32 elements from LDS, B = the wavefront's queries, kept in registers
 //   O^T = V^T P^T   A = 16 elements x 32 keys from the transposed copy, B = the probabilities just computed
@@ -47,8 +48,6 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   const int k_stride = dk_steps * 32 + kLmPad;                 // elements
   const int v_tiles = (rank + 15) / 16;
   constexpr int v_stride = kLmKeys + kLmPad;
-  bf16* k_lds = reinterpret_cast<bf16*>(lds_raw);              // [32][k_stride]
-  bf16* v_lds = k_lds + kLmKeys * k_stride;                    // [v_tiles * 16][v_stride]
 
   const int seq = seq_ids ? seq_ids[blockIdx.y] : blockIdx.y;
   const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
@@ -99,70 +98,105 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   for (int t = 0; t < RT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const float c = scale * kLog2eL;
-  const int chunks = dk_steps * 4;                             // 16-byte pieces of a staged row
   const bool wave_active = rb + wave * 16 < rows;              // a wavefront without rows of its own only helps staging
 
-  // A block's pieces, a thread's share held in registers between their loads and their stores into LDS, so that the
-  // loads of the next block are in flight while this block is worked on.  Rows: piece i is key i % 32, elements
-  // 8 (i / 32)...; the transposed copy: piece i is element i / 4, keys 8 (i % 4)... (pages hold multiples of 8 keys,
-  // so eight keys from a multiple of 8 lie in one page).
-  constexpr int KC = (kLmKeys * QS * 4 + 255) / 256;
-  constexpr int VC = (RT * 16 * 4 + 255) / 256;
-  bf16x8 kreg[KC], vreg[VC];
-  auto load_block = [&](int b0) {
+  // Staging goes from memory straight into LDS (no registers in between: with the queries and the output tiles a
+  // wavefront holds, staged pieces parked in registers were waited for one by one).  One such load fills 64
+  // consecutive 16-byte pieces of LDS, a piece a lane, from 64 addresses of the lanes' own; the two regions are
+  // laid out piece by piece: rows of k_pieces (a row's pieces and one of padding), then the transposed copy's rows
+  // of five (four runs of 8 keys and one of padding).  Pieces of padding, keys past the range and pages given back
+  // are loaded from clamped addresses: what they bring is finite and is masked or multiplied by zero.  Two buffers:
+  // the next block's loads are in flight while this block is worked on.
+  const int k_pieces = dk_steps * 4 + 1;
+  const int k_loads = (kLmKeys * k_pieces + 63) / 64, v_loads = (v_tiles * 16 * 5 + 63) / 64;
+  const int buf_elems = (k_loads + v_loads) * 512;             // 64 pieces of 8 elements a load
+  const int ch_last = dk / 8 - 1;
+  // Where this lane's piece of each load lies does not change from block to block: piece i = 64 * load + lane of
+  // the rows is key i / k_pieces, piece i % k_pieces; the loads of a wavefront are 256 pieces apart, so the pair is
+  // stepped, not divided, and the divisions happen once.
+  const int k_step_key = 256 / k_pieces, k_step_ch = 256 % k_pieces;
+  const int k_key0 = (wave * 64 + lane) / k_pieces, k_ch0 = (wave * 64 + lane) % k_pieces;
+  auto issue_block = [&](int b0, bf16* buf) {
+    const int last = end_wg - 1;
+    const int rel_last = last - b0;                              // >= 0: the block holds a key of the range
+    // the pages of the block's four runs of 8 keys (pages hold multiples of 8 keys) and the runs' places in them
+    size_t row0[4], run0[4];                                     // first row of a run in the cache; the run in the copy
 #pragma unroll
-    for (int cI = 0; cI < KC; ++cI) {
-      const int i = threadIdx.x + 256 * cI;
-      const int key = i % kLmKeys, ch = i / kLmKeys;
-      const int kidx = b0 + key;
-      bf16x8 v = {};
-      if (ch < chunks && kidx < end_wg && 8 * ch + 8 <= dk) {
-        const int page = table[kidx / page_size];
-        if (page >= 0) v = *reinterpret_cast<const bf16x8*>(cache + ((size_t)page * page_size + kidx % page_size) * dk + 8 * ch);
+    for (int j = 0; j < 4; ++j) {
+      const int kc = 8 * j <= rel_last ? b0 + 8 * j : (last & ~7);
+      const int at = kc / page_size;
+      const int page = table[at];
+      const size_t pg = page >= 0 ? page : 0, place = kc - at * page_size;
+      row0[j] = pg * page_size + place;
+      run0[j] = pg * rank * page_size + place;
+    }
+    int key = k_key0, ch = k_ch0;
+    for (int sI = wave; sI < k_loads; sI += 4) {
+      int kk = key < kLmKeys ? key : kLmKeys - 1;
+      kk = kk < rel_last ? kk : rel_last;
+      const int j = kk >> 3;
+      const size_t row = (j == 0 ? row0[0] : (j == 1 ? row0[1] : (j == 2 ? row0[2] : row0[3]))) + (kk & 7);
+      const bf16* src = cache + row * dk + 8 * (ch < ch_last ? ch : ch_last);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(buf + (size_t)sI * 512), 16, 0, 0);
+      key += k_step_key;
+      ch += k_step_ch;
+      if (ch >= k_pieces) {
+        ch -= k_pieces;
+        ++key;
       }
-      kreg[cI] = v;
     }
-#pragma unroll
-    for (int cI = 0; cI < VC; ++cI) {
-      const int i = threadIdx.x + 256 * cI;
-      const int vrow = i / 4, kidx = b0 + 8 * (i % 4);
-      bf16x8 v = {};
-      if (vrow < rank && kidx < end_wg) {
-        const int page = table[kidx / page_size];
-        if (page >= 0) v = *reinterpret_cast<const bf16x8*>(cache_t + ((size_t)page * rank + vrow) * page_size + kidx % page_size);
-      }
-      vreg[cI] = v;
-    }
-  };
-  auto store_block = [&]() {
-#pragma unroll
-    for (int cI = 0; cI < KC; ++cI) {
-      const int i = threadIdx.x + 256 * cI;
-      if (i / kLmKeys < chunks) *reinterpret_cast<bf16x8*>(k_lds + (i % kLmKeys) * k_stride + 8 * (i / kLmKeys)) = kreg[cI];
-    }
-#pragma unroll
-    for (int cI = 0; cI < VC; ++cI) {
-      const int i = threadIdx.x + 256 * cI;
-      if (i / 4 < v_tiles * 16) *reinterpret_cast<bf16x8*>(v_lds + (i / 4) * v_stride + 8 * (i % 4)) = vreg[cI];
+    // the transposed copy: piece i is element i / 5, run i % 5 (the fifth is padding)
+    for (int sI = wave; sI < v_loads; sI += 4) {
+      const int i = sI * 64 + lane;
+      int vrow = i / 5, j = i % 5;
+      vrow = vrow < rank ? vrow : rank - 1;
+      j = (j < 4 && 8 * j <= rel_last) ? j : 0;
+      const size_t r0 = j == 0 ? run0[0] : (j == 1 ? run0[1] : (j == 2 ? run0[2] : run0[3]));
+      const bf16* src = cache_t + r0 + (size_t)vrow * page_size;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(buf + (size_t)(k_loads + sI) * 512), 16, 0, 0);
     }
   };
 
-  if (lo_wg < end_wg) load_block(lo_wg);
-  for (int b0 = lo_wg; b0 < end_wg; b0 += kLmKeys) {
-    __syncthreads();
-    store_block();
-    __syncthreads();
-    if (b0 + kLmKeys < end_wg) load_block(b0 + kLmKeys);
+  bf16* const buf0 = reinterpret_cast<bf16*>(lds_raw);
+  if (lo_wg < end_wg) issue_block(lo_wg, buf0);
+  int it = 0;
+  for (int b0 = lo_wg; b0 < end_wg; b0 += kLmKeys, ++it) {
+    bf16* const cur = buf0 + (it & 1) * buf_elems;
+    __builtin_amdgcn_s_waitcnt(0);                             // this wavefront's share of the block has landed
+    __syncthreads();                                           // ... and everyone's; all are done with the other buffer
+    if (b0 + kLmKeys < end_wg) issue_block(b0 + kLmKeys, buf0 + ((it + 1) & 1) * buf_elems);
     if (!wave_active) continue;
+    const bf16* k_lds = cur;
+    const bf16* v_lds = cur + k_loads * 512;
     // ---- scores of 32 keys for this wavefront's 16 rows ----
+    // Operands are read from LDS in batches ahead of the products that use them (a wavefront is alone on its SIMD:
+    // a read waited for right before its product costs the LDS's latency every time), and the two tiles' chains of
+    // dependent products run interleaved.
     f32x4 s[2];
+    s[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    {
+      const bf16* kr0 = k_lds + (8 * (r / 4) + (r % 4)) * k_stride + 8 * g;
+      const bf16* kr1 = kr0 + 4 * k_stride;
+      constexpr int kBatch = 6;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const bf16* kr = k_lds + (8 * (r / 4) + 4 * t + (r % 4)) * k_stride + 8 * g;
+      for (int k0 = 0; k0 < QS; k0 += kBatch) {
+        bf16x8 ka[kBatch], kb[kBatch];
 #pragma unroll
-      for (int ks = 0; ks < QS; ++ks) {
-        if (ks < dk_steps) s[t] = mfma16l(*reinterpret_cast<const bf16x8*>(kr + 32 * ks), qf[ks], s[t]);
+        for (int j = 0; j < kBatch; ++j) {
+          const int ks = k0 + j < QS ? k0 + j : QS - 1;      // (a step past the latent's own reads inside the buffer and is not used)
+          ka[j] = *reinterpret_cast<const bf16x8*>(kr0 + 32 * (ks < dk_steps ? ks : 0));
+          kb[j] = *reinterpret_cast<const bf16x8*>(kr1 + 32 * (ks < dk_steps ? ks : 0));
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+          if (k0 + j < QS && k0 + j < dk_steps) {
+            s[0] = mfma16l(ka[j], qf[k0 + j], s[0]);
+            s[1] = mfma16l(kb[j], qf[k0 + j], s[1]);
+          }
+        }
       }
     }
     // ---- mask, running maximum, probabilities ----
@@ -194,11 +228,28 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     l = l * alpha + psum;
     m = m_new;
     // ---- weighted sum: O^T += V^T P^T ----
+    // (the sums are rescaled only in blocks where some row's maximum moved: early ones, and rarely later)
+    const bool rescale = __any(alpha != 1.0f);
+    {
+      const bf16* vr = v_lds + r * v_stride + 8 * g;
+      constexpr int vBatch = 8;
 #pragma unroll
-    for (int t = 0; t < RT; ++t) {
-      if (t < v_tiles) {
-        o[t] *= alpha;
-        o[t] = mfma16l(*reinterpret_cast<const bf16x8*>(v_lds + (16 * t + r) * v_stride + 8 * g), pf, o[t]);
+      for (int t0 = 0; t0 < RT; t0 += vBatch) {
+        if (t0 < v_tiles) {
+          bf16x8 vf[vBatch];
+#pragma unroll
+          for (int j = 0; j < vBatch; ++j) {
+            const int t = t0 + j < RT ? t0 + j : RT - 1;
+            vf[j] = *reinterpret_cast<const bf16x8*>(vr + 16 * (t < v_tiles ? t : 0) * v_stride);
+          }
+#pragma unroll
+          for (int j = 0; j < vBatch; ++j) {
+            if (t0 + j < RT && t0 + j < v_tiles) {
+              if (rescale) o[t0 + j] *= alpha;
+              o[t0 + j] = mfma16l(vf[j], pf, o[t0 + j]);
+            }
+          }
+        }
       }
     }
   }
@@ -297,7 +348,8 @@ static int launch_latent_mfma(hipStream_t st, dim3 grid, size_t lds, const bf16*
 
 static size_t latent_mfma_lds(int rank, int rot) {
   const int dk_steps = (rank + rot + 31) / 32, v_tiles = (rank + 15) / 16;
-  return (size_t)(kLmKeys * (dk_steps * 32 + kLmPad) + v_tiles * 16 * (kLmKeys + kLmPad)) * sizeof(bf16);
+  const int k_loads = (kLmKeys * (dk_steps * 4 + 1) + 63) / 64, v_loads = (v_tiles * 16 * 5 + 63) / 64;
+  return (size_t)2 * (k_loads + v_loads) * 1024;               // two buffers of whole 64-piece loads
 }
 
 }  // namespace pa
