@@ -3,7 +3,7 @@
 // (group = head, rows = tokens).
 //
 // y[row, n] = sum_k x[row, k] * w[group, n, k], the weight as stored ([out, in], in fastest).  A workgroup of four
-// wavefronts owns up to 64 rows of one group and 128 outputs: each wavefront two tiles of 16 outputs against the
+// wavefronts owns up to 64 rows of one group and 256 outputs: each wavefront four tiles of 16 outputs against the
 // four tiles of 16 rows, W^T tile as A (row = output), X^T as B (column = row of x), both straight from memory in
 // 16-byte pieces (v_mfma_f32_16x16x32_bf16: A row r, columns 8g..8g+7; B column r, rows 8g..8g+7; C column r,
 // rows 4g..4g+3).  A weight element is read once per 64 rows, and sums run over k in ascending steps of 32
@@ -14,7 +14,8 @@
 namespace pa {
 
 constexpr int kGmRows = 64;
-constexpr int kGmCols = 128;
+constexpr int kGmCols = 256;
+constexpr int kGmWaveTiles = 4;   // tiles of 16 outputs a wavefront
 
 // xrow(m) / yrow(m): element offsets of row m's input and output, < 0 for a row that does not exist.
 template <typename TY, typename RowX, typename RowY>
@@ -23,42 +24,42 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int row_tiles = (n_rows + 15) / 16;
-  long xo[4];
+  // Every load is unconditional (rows, outputs and the last step of k that do not exist are clamped to ones that do:
+  // loads under branches are waited for one by one); what a clamped row or output brings is never stored, and the
+  // one thing that must not count, a step past the end of k, is zeroed on the x side by a select.
+  const bf16* xr[4];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) xo[mt] = (mt * 16 + r < n_rows) ? xrow(mt * 16 + r) : -1;
-  const int nb = n0 + wave * 32;
-  const bf16* wr[2];
-  bool wok[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = nb + 16 * j + r;
-    wok[j] = n < N;
-    wr[j] = w + (size_t)(wok[j] ? n : 0) * K + 8 * g;
-  }
+  for (int mt = 0; mt < 4; ++mt) xr[mt] = x + xrow(mt * 16 + r < n_rows ? mt * 16 + r : 0) + 8 * g;
+  constexpr int NT = kGmWaveTiles;
+  const int nb = n0 + wave * 16 * NT;
   if (nb >= N) return;
-  f32x4 acc[2][4];
+  const bf16* wr[NT];
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < NT; ++j) {
+    const int n = nb + 16 * j + r;
+    wr[j] = w + (size_t)(n < N ? n : N - 1) * K + 8 * g;
+  }
+  f32x4 acc[NT][4];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[j][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < K; k0 += 32) {
     const bool kok = k0 + 8 * g + 8 <= K;
-    bf16x8 wf[2], xf[4];
+    const int kc = kok ? k0 : K - 8 - 8 * g;                    // (K is a multiple of 8: the clamped piece lies inside the row)
+    bf16x8 wf[NT], xf[4];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      wf[j] = bf16x8{};
-      if (kok && wok[j]) wf[j] = *reinterpret_cast<const bf16x8*>(wr[j] + k0);
-    }
+    for (int j = 0; j < NT; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(wr[j] + kc);
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
-      xf[mt] = bf16x8{};
-      if (mt < row_tiles && kok && xo[mt] >= 0) xf[mt] = *reinterpret_cast<const bf16x8*>(x + xo[mt] + k0 + 8 * g);
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(xr[mt < row_tiles ? mt : 0] + kc);
+      xf[mt] = kok ? v : bf16x8{};
     }
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       if (mt < row_tiles) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[mt], acc[j][mt], 0, 0, 0);
+        for (int j = 0; j < NT; ++j) acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[mt], acc[j][mt], 0, 0, 0);
       }
     }
   }
@@ -68,7 +69,7 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
     const long yo = yrow(mt * 16 + r);
     if (yo < 0) continue;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int n = nb + 16 * j + 4 * g + i;
