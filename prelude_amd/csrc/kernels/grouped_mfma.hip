@@ -3,7 +3,7 @@
 // (group = head, rows = tokens).
 //
 // y[row, n] = sum_k x[row, k] * w[group, n, k], the weight as stored ([out, in], in fastest).  A workgroup of four
-// wavefronts owns up to 64 rows of one group and 256 outputs: each wavefront four tiles of 16 outputs against the
+// wavefronts owns up to 64 rows of one group and 256 (or 128) outputs: each wavefront four (two) tiles of 16 outputs against the
 // four tiles of 16 rows, W^T tile as A (row = output), X^T as B (column = row of x), both straight from memory in
 // 16-byte pieces (v_mfma_f32_16x16x32_bf16: A row r, columns 8g..8g+7; B column r, rows 8g..8g+7; C column r,
 // rows 4g..4g+3).  A weight element is read once per 64 rows, and sums run over k in ascending steps of 32
@@ -14,11 +14,11 @@
 namespace pa {
 
 constexpr int kGmRows = 64;
-constexpr int kGmCols = 256;
-constexpr int kGmWaveTiles = 4;   // tiles of 16 outputs a wavefront
+// tiles of 16 outputs a wavefront: four where there are rows enough to reuse them (a workgroup then owns 256 outputs),
+// two for the few rows of a step of single tokens, where what counts is how many workgroups stream the weights (128)
 
 // xrow(m) / yrow(m): element offsets of row m's input and output, < 0 for a row that does not exist.
-template <typename TY, typename RowX, typename RowY>
+template <typename TY, int NT, typename RowX, typename RowY>
 __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const bf16* __restrict__ w, TY* __restrict__ y,
                                              int K, int N, int n_rows, int n0, int act, RowX xrow, RowY yrow) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -30,7 +30,6 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
   const bf16* xr[4];
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) xr[mt] = x + xrow(mt * 16 + r < n_rows ? mt * 16 + r : 0) + 8 * g;
-  constexpr int NT = kGmWaveTiles;
   const int nb = n0 + wave * 16 * NT;
   if (nb >= N) return;
   const bf16* wr[NT];
@@ -87,7 +86,7 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
 
 // Experts: blockIdx.x walks the tiles of 64 positions of all experts in order (an expert with c entries has
 // ceil(c / 64) tiles; blocks beyond the last leave).  `from_tokens`: position p reads row order[p] / top of x.
-template <typename TY>
+template <typename TY, int NT>
 __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                              TY* __restrict__ y, const int* __restrict__ offsets,
                                                              const int* __restrict__ order, int experts, int top, int K,
@@ -104,18 +103,19 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __rest
     tile -= tiles;
   }
   if (e >= experts) return;
-  grouped_tile<TY>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, blockIdx.y * kGmCols, act,
+  grouped_tile<TY, NT>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, blockIdx.y * 64 * NT, act,
                    [&](int m) { return (long)(from_tokens ? order[p0 + m] / top : p0 + m) * K; },
                    [&](int m) { return (long)(p0 + m) * N; });
 }
 
-// Heads: grid (tiles of 64 tokens, heads, chunks of 128 outputs).
+// Heads: grid (tiles of 64 tokens, heads, chunks of 64 NT outputs).
+template <int NT>
 __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                               bf16* __restrict__ y, int tokens, int K, int N, long xs_t,
                                                               long xs_h, long ys_t, long ys_h) {
   const int t0 = blockIdx.x * kGmRows, h = blockIdx.y;
   const int n_rows = tokens - t0 < kGmRows ? tokens - t0 : kGmRows;
-  grouped_tile<bf16>(x, w + (size_t)h * N * K, y, K, N, n_rows, blockIdx.z * kGmCols, 0,
+  grouped_tile<bf16, NT>(x, w + (size_t)h * N * K, y, K, N, n_rows, blockIdx.z * 64 * NT, 0,
                      [&](int m) { return (long)(t0 + m) * xs_t + (long)h * xs_h; },
                      [&](int m) { return (long)(t0 + m) * ys_t + (long)h * ys_h; });
 }
@@ -132,16 +132,21 @@ extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, cons
   PA_REQUIRE(entries > 0 && experts > 0 && top > 0 && K > 0 && N > 0 && K % 8 == 0, "moe_linear_mfma: bad sizes entries=%d experts=%d k=%d n=%d",
              entries, experts, K, N);
   PA_REQUIRE(act == 0 || act == 1, "moe_linear_mfma: unknown activation code %d", act);
-  dim3 grid((entries + kGmRows - 1) / kGmRows + experts, (N + kGmCols - 1) / kGmCols);
+  const bool few = entries <= 4 * kGmRows;
+  const int cols = few ? 128 : 256;
+  dim3 grid((entries + kGmRows - 1) / kGmRows + experts, (N + cols - 1) / cols);
   hipStream_t st = (hipStream_t)stream;
-  if (y_dtype == kBF16)
-    hipLaunchKernelGGL(moe_linear_mfma_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (bf16*)y, offsets, order,
-                       experts, top, K, N, from_tokens, act);
-  else if (y_dtype == kF32)
-    hipLaunchKernelGGL(moe_linear_mfma_kernel<float>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (float*)y, offsets, order,
-                       experts, top, K, N, from_tokens, act);
-  else
+#define PA_GM(TY, NT)                                                                                                       \
+  hipLaunchKernelGGL((moe_linear_mfma_kernel<TY, NT>), grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (TY*)y, offsets, \
+                     order, experts, top, K, N, from_tokens, act)
+  if (y_dtype == kBF16) {
+    if (few) PA_GM(bf16, 2); else PA_GM(bf16, 4);
+  } else if (y_dtype == kF32) {
+    if (few) PA_GM(float, 2); else PA_GM(float, 4);
+  } else {
     return pa::fail("moe_linear_mfma: unknown output type code %d", y_dtype);
+  }
+#undef PA_GM
   return check_launch("moe_linear_mfma");
 }
 
@@ -152,9 +157,15 @@ extern "C" int pa_head_linear_mfma(void* stream, const void* x, const void* w, v
   PA_REQUIRE(tokens > 0 && heads > 0 && K > 0 && N > 0 && K % 8 == 0 && xs_t % 8 == 0 && xs_h % 8 == 0,
              "head_linear_mfma: bad sizes tokens=%d heads=%d k=%d n=%d strides %ld %ld", tokens, heads, K, N, xs_t, xs_h);
   PA_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0, "head_linear_mfma: operands are not 16-byte aligned");
-  PA_REQUIRE(heads <= 65535 && (N + kGmCols - 1) / kGmCols <= 65535, "head_linear_mfma: %d heads or %d outputs exceed the grid", heads, N);
-  dim3 grid((tokens + kGmRows - 1) / kGmRows, heads, (N + kGmCols - 1) / kGmCols);
-  hipLaunchKernelGGL(head_linear_mfma_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, (const bf16*)w, (bf16*)y, tokens,
-                     K, N, xs_t, xs_h, ys_t, ys_h);
+  const bool few = tokens <= kGmRows;
+  const int cols = few ? 128 : 256;
+  PA_REQUIRE(heads <= 65535 && (N + cols - 1) / cols <= 65535, "head_linear_mfma: %d heads or %d outputs exceed the grid", heads, N);
+  dim3 grid((tokens + kGmRows - 1) / kGmRows, heads, (N + cols - 1) / cols);
+  if (few)
+    hipLaunchKernelGGL(head_linear_mfma_kernel<2>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, (const bf16*)w, (bf16*)y,
+                       tokens, K, N, xs_t, xs_h, ys_t, ys_h);
+  else
+    hipLaunchKernelGGL(head_linear_mfma_kernel<4>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, (const bf16*)w, (bf16*)y,
+                       tokens, K, N, xs_t, xs_h, ys_t, ys_h);
   return check_launch("head_linear_mfma");
 }

@@ -301,30 +301,52 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 }
 
 // out[row] = sum over the splits' partials, each scaled by exp(its maximum - the largest), then the sink.
-// One workgroup a row; the splits are added in order.
+// One workgroup a row; the splits' factors are worked out once (in LDS), then every thread adds its elements over
+// the splits in order, eight loads in flight.
+constexpr int kMergeMaxSplits = 4096;
 __global__ __launch_bounds__(256) void latent_attn_merge_kernel(const float* __restrict__ ws, const float* __restrict__ sink,
                                                                const int* __restrict__ seq_ids, const int* __restrict__ cu_q,
                                                                bf16* __restrict__ out, int nh, int rank, int n_splits) {
+  __shared__ float factor[kMergeMaxSplits];
+  __shared__ float scratch[16];
   const int row = blockIdx.x;                                  // (place in the launch) * heads + head
   const int seq = seq_ids ? seq_ids[row / nh] : row / nh;
   const size_t out_row = (size_t)cu_q[seq] * nh + row % nh;
-  const float* w = ws + (size_t)row * n_splits * (rank + 2);
+  const size_t stride = (size_t)rank + 2;
+  const float* w = ws + (size_t)row * n_splits * stride;
   float top = -INFINITY;
-  for (int z = 0; z < n_splits; ++z) top = fmaxf(top, w[(size_t)z * (rank + 2)]);
+  for (int z = threadIdx.x; z < n_splits; z += blockDim.x) top = fmaxf(top, w[z * stride]);
+  top = wave_max(top);
+  {
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    if (lane == 0) scratch[wave] = top;
+    __syncthreads();
+    for (int i = 0; i < (int)(blockDim.x / kWave); ++i) top = fmaxf(top, scratch[i]);
+    __syncthreads();
+  }
   const float sk = sink ? sink[row % nh] : -INFINITY;
   top = fmaxf(top, sk);
-  float l = sink ? expf(sk - top) : 0.f;
-  for (int z = 0; z < n_splits; ++z) {
-    const float mz = w[(size_t)z * (rank + 2)];
-    if (mz != -INFINITY) l += w[(size_t)z * (rank + 2) + 1] * expf(mz - top);
+  float lpart = 0.f;
+  for (int z = threadIdx.x; z < n_splits; z += blockDim.x) {
+    const float mz = w[z * stride];
+    const float f = mz == -INFINITY ? 0.f : expf(mz - top);
+    factor[z] = f;
+    lpart += f * w[z * stride + 1];
   }
+  float l = block_sum(lpart, scratch);                         // (its barriers also publish the factors)
+  if (sink) l += expf(sk - top);
   const float inv = 1.f / l;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     float acc = 0.f;
-    for (int z = 0; z < n_splits; ++z) {
-      const float mz = w[(size_t)z * (rank + 2)];
-      if (mz != -INFINITY) acc += w[(size_t)z * (rank + 2) + 2 + d] * expf(mz - top);
+    int z = 0;
+    for (; z + 8 <= n_splits; z += 8) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = w[(z + j) * stride + 2 + d];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc += v[j] * factor[z + j];
     }
+    for (; z < n_splits; ++z) acc += w[z * stride + 2 + d] * factor[z];
     out[out_row * rank + d] = (bf16)(acc * inv);
   }
 }
@@ -381,6 +403,7 @@ extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cach
              "latent_attn_mfma: bad sizes seqs=%d q=%d heads=%d stride=%d window=%d", n_seqs, max_q_len, nh, table_stride, window);
   PA_REQUIRE(cache && cache_t, "latent_attn_mfma: needs the cache and its transposed copy");
   PA_REQUIRE(scale > 0.f, "latent_attn_mfma: a scale of %g is not positive", (double)scale);
+  PA_REQUIRE(n_splits <= kMergeMaxSplits, "latent_attn_mfma: %d splits are more than the %d the merge takes", n_splits, kMergeMaxSplits);
   PA_REQUIRE(n_splits >= 1 && (n_splits == 1 || (split_keys > 0 && split_keys % kLmKeys == 0 && ws && max_q_len == 1)),
              "latent_attn_mfma: %d splits of %d keys need a workspace, whole blocks and sequences of one token", n_splits, split_keys);
   const long tiles = ((long)max_q_len * nh + kLmRows - 1) / kLmRows;

@@ -86,6 +86,35 @@ __global__ void relu_squared_kernel(const T* __restrict__ x, T* __restrict__ out
   out[i] = from_f32<T>(v * v);
 }
 
+// The same in 16-byte pieces for bfloat16: a thread takes eight pairs (two loads) and writes eight outputs.
+__global__ void clamped_gate_vec_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, size_t groups, float limit,
+                                        float alpha) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= groups) return;
+  const bf16x8 a = *reinterpret_cast<const bf16x8*>(gate_up + 16 * i);
+  const bf16x8 b = *reinterpret_cast<const bf16x8*>(gate_up + 16 * i + 8);
+  bf16x8 o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    o[j] = (bf16)clamped_gate((float)a[2 * j], (float)a[2 * j + 1], limit, alpha);
+    o[4 + j] = (bf16)clamped_gate((float)b[2 * j], (float)b[2 * j + 1], limit, alpha);
+  }
+  *reinterpret_cast<bf16x8*>(out + 8 * i) = o;
+}
+
+__global__ void relu_squared_vec_kernel(const bf16* __restrict__ x, bf16* __restrict__ out, size_t groups) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= groups) return;
+  const bf16x8 a = *reinterpret_cast<const bf16x8*>(x + 8 * i);
+  bf16x8 o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float v = fmaxf((float)a[j], 0.f);
+    o[j] = (bf16)(v * v);
+  }
+  *reinterpret_cast<bf16x8*>(out + 8 * i) = o;
+}
+
 template <typename T>
 static void launch_wide(hipStream_t st, const T* x, const float* parts, int slices, size_t slice_stride, float* residual,
                         const float* w, T* out, const int* rows, int nrows, int hidden, float eps) {
@@ -130,6 +159,11 @@ extern "C" int pa_clamped_gate(void* stream, int dtype, const void* gate_up, voi
   const size_t total = (size_t)tokens * inter;
   const unsigned blocks = (unsigned)((total + 255) / 256);
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == kBF16 && total % 8 == 0 && ((uintptr_t)gate_up & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    hipLaunchKernelGGL(clamped_gate_vec_kernel, dim3((unsigned)((total / 8 + 255) / 256)), dim3(256), 0, st, (const bf16*)gate_up,
+                       (bf16*)out, total / 8, limit, alpha);
+    return check_launch("clamped_gate");
+  }
   if (dtype == kF32)
     hipLaunchKernelGGL(clamped_gate_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)gate_up, (float*)out, total, limit, alpha);
   else if (dtype == kBF16)
@@ -144,6 +178,11 @@ extern "C" int pa_relu_squared(void* stream, int dtype, const void* x, void* out
   PA_REQUIRE(total > 0, "relu_squared: bad size %ld", total);
   const unsigned blocks = (unsigned)((total + 255) / 256);
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == kBF16 && total % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    hipLaunchKernelGGL(relu_squared_vec_kernel, dim3((unsigned)((total / 8 + 255) / 256)), dim3(256), 0, st, (const bf16*)x, (bf16*)out,
+                       (size_t)(total / 8));
+    return check_launch("relu_squared");
+  }
   if (dtype == kF32)
     hipLaunchKernelGGL(relu_squared_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)x, (float*)out, (size_t)total);
   else if (dtype == kBF16)

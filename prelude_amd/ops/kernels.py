@@ -1270,7 +1270,22 @@ def moe_combine(y: torch.Tensor, eo: ExpertOrder, weight: float, base: Optional[
 LATENT_MAX_WIDTH = 1024   # rank + rot of a cached latent vector the attention kernels take
 
 
-LATENT_SPLIT_KEYS = 256    # keys a split of the matrix-core kernel, for steps of single tokens
+# Keys a split of the matrix-core kernel, for steps of single tokens: a workgroup walks its split block by block, one
+# after the other, so the shortest split that still leaves the launch within LATENT_SPLIT_WORKGROUPS workgroups is the
+# fastest (8 sequences of 4,096 keys: 512 workgroups of 2 blocks instead of 128 of 8)
+LATENT_SPLIT_KEYS = (64, 128, 256)
+LATENT_SPLIT_WORKGROUPS = 768
+LATENT_MAX_SPLITS = 4096     # what the merge kernel takes; contexts beyond 4,096 splits of 256 keys get longer splits
+
+
+def latent_split_keys(n_seqs: int, max_context: int) -> int:
+    for keys in LATENT_SPLIT_KEYS:
+        if n_seqs * -(-int(max_context) // keys) <= LATENT_SPLIT_WORKGROUPS:
+            return keys
+    keys = LATENT_SPLIT_KEYS[-1]
+    while -(-int(max_context) // keys) > LATENT_MAX_SPLITS:
+        keys *= 2
+    return keys
 
 
 def latent_attention_mfma_supported(rank: int, rot: int, page_size: int) -> bool:
@@ -1283,7 +1298,7 @@ def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, cache_t: torch.T
                           max_context: int = 0) -> None:
     """The matrix-core kernel for the sequences ``seq_ids`` (None: all ``n_seqs`` of the step); writes their rows of
     ``out`` [T, heads, rank].  ``max_context`` > 0 with ``max_q_len`` 1 cuts the keys into splits of
-    ``LATENT_SPLIT_KEYS`` whose partials a second kernel merges: what fills the chip when every sequence feeds one token."""
+    ``latent_split_keys`` keys whose partials a second kernel merges: what fills the chip when every sequence feeds one token."""
     _dev(q, cache, cache_t, sink, block_table, seq_ids, cu_q, context_lens, out)
     _f32(sink, "sink")
     t, nh, dk = q.shape
@@ -1295,13 +1310,14 @@ def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, cache_t: torch.T
     if n_seqs == 0:
         return
     splits, ws = 1, None
-    if max_q_len == 1 and max_context > LATENT_SPLIT_KEYS:
-        splits = -(-int(max_context) // LATENT_SPLIT_KEYS)
+    split_keys = latent_split_keys(n_seqs, max_context)
+    if max_q_len == 1 and max_context > split_keys:
+        splits = -(-int(max_context) // split_keys)
         ws = torch.empty(int(kernels().pa_latent_attn_mfma_workspace(n_seqs, nh, rank, splits)), dtype=torch.float32, device=q.device)
     check(kernels().pa_latent_attn_mfma(_stream(), _ptr(q), _ptr(cache), _ptr(cache_t), _ptr(sink), _ptr(block_table), block_table.shape[1],
                                         _ptr(seq_ids), _ptr(cu_q), _ptr(context_lens), _ptr(out), _ptr(ws), int(n_seqs),
                                         int(max_q_len), nh, int(rank), dk - int(rank), cache.shape[1], int(window), float(scale),
-                                        LATENT_SPLIT_KEYS, splits))
+                                        split_keys, splits))
 
 
 def latent_attention(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], group, step, rank: int,

@@ -62,13 +62,14 @@ def test_norm_with_a_32_bit_residual(gpu, dtype, hidden):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_clamped_pair_and_squared_relu(gpu, dtype):
     from prelude_amd.ops import kernels as K
-    gu = rnd((9, 2 * 37), 5, dtype, 2.0)
-    g, u = gu[:, 0::2].double(), gu[:, 1::2].double()
-    for limit, alpha in ((1.5, 1.702), (0.4, 1.0), (7.0, 2.5)):
-        gc, uc = torch.clamp(g, max=limit), torch.clamp(u, -limit, limit)
-        close(K.clamped_gate(gu.to(gpu), limit, alpha), gc * torch.sigmoid(alpha * gc) * (uc + 1), dtype, f"limit {limit}")
-    x = rnd((5, 33), 6, dtype)
-    close(K.relu_squared(x.to(gpu)), torch.relu(x.double()) ** 2, dtype, "squared relu")
+    for rows, inter in ((9, 37), (8, 40)):       # (the second: whole 16-byte pieces, the vector kernels' case)
+        gu = rnd((rows, 2 * inter), 5, dtype, 2.0)
+        g, u = gu[:, 0::2].double(), gu[:, 1::2].double()
+        for limit, alpha in ((1.5, 1.702), (0.4, 1.0), (7.0, 2.5)):
+            gc, uc = torch.clamp(g, max=limit), torch.clamp(u, -limit, limit)
+            close(K.clamped_gate(gu.to(gpu), limit, alpha), gc * torch.sigmoid(alpha * gc) * (uc + 1), dtype, f"limit {limit}")
+        x = rnd((rows, inter), 6, dtype)
+        close(K.relu_squared(x.to(gpu)), torch.relu(x.double()) ** 2, dtype, "squared relu")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
