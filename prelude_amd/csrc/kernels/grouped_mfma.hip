@@ -43,23 +43,37 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[j][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < K; k0 += 32) {
+  // The operands of the step after this one are asked for before this step's products, into a second set of
+  // registers: a step's loads take far longer than its products, and this keeps two steps' worth in flight.
+  bf16x8 wf[2][NT], xf[2][4];
+  auto load_step = [&](int k0, int b) {
     const bool kok = k0 + 8 * g + 8 <= K;
     const int kc = kok ? k0 : K - 8 - 8 * g;                    // (K is a multiple of 8: the clamped piece lies inside the row)
-    bf16x8 wf[NT], xf[4];
 #pragma unroll
-    for (int j = 0; j < NT; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(wr[j] + kc);
+    for (int j = 0; j < NT; ++j) wf[b][j] = *reinterpret_cast<const bf16x8*>(wr[j] + kc);
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       const bf16x8 v = *reinterpret_cast<const bf16x8*>(xr[mt < row_tiles ? mt : 0] + kc);
-      xf[mt] = kok ? v : bf16x8{};
+      xf[b][mt] = kok ? v : bf16x8{};
     }
+  };
+  auto multiply = [&](int b) {
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       if (mt < row_tiles) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[mt], acc[j][mt], 0, 0, 0);
+        for (int j = 0; j < NT; ++j) acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[b][j], xf[b][mt], acc[j][mt], 0, 0, 0);
       }
+    }
+  };
+  const int last_k0 = ((K - 1) / 32) * 32;
+  load_step(0, 0);
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    load_step(k0 + 32 <= last_k0 ? k0 + 32 : last_k0, 1);      // (past the end: the last step once more, not multiplied)
+    multiply(0);
+    if (k0 + 32 < K) {
+      load_step(k0 + 64 <= last_k0 ? k0 + 64 : last_k0, 0);
+      multiply(1);
     }
   }
 #pragma unroll
@@ -89,9 +103,19 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
 template <typename TY, int NT>
 __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                              TY* __restrict__ y, const int* __restrict__ offsets,
-                                                             const int* __restrict__ order, int experts, int top, int K,
-                                                             int N, int from_tokens, int act) {
-  int tile = blockIdx.x, e = 0, p0 = 0, p1 = 0;
+                                                             const int* __restrict__ order, int entries, int experts,
+                                                             int top, int K, int N, int col_chunks, int from_tokens, int act) {
+  // The launch is a line of workgroups that the hardware deals out to the eight XCDs in turn (each with an L2 of
+  // its own); work item w = (chunk of outputs, tile of positions), tiles fastest, and every XCD is given one stretch
+  // of the items: the tiles of one expert against one chunk of its weight then run on one XCD one after the other,
+  // and the chunk comes from memory once instead of once a tile.
+  const int tiles_max = (entries + kGmRows - 1) / kGmRows + experts;
+  const int total = tiles_max * col_chunks;
+  const int per_xcd = (total + 7) / 8;
+  const int item = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+  if (blockIdx.x / 8 >= (unsigned)per_xcd || item >= total) return;
+  int tile = item % tiles_max, e = 0, p0 = 0, p1 = 0;
+  const int col_chunk = item / tiles_max;
   for (; e < experts; ++e) {
     const int a = offsets[e], b = offsets[e + 1];
     const int tiles = (b - a + kGmRows - 1) / kGmRows;
@@ -103,7 +127,7 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __rest
     tile -= tiles;
   }
   if (e >= experts) return;
-  grouped_tile<TY, NT>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, blockIdx.y * 64 * NT, act,
+  grouped_tile<TY, NT>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, col_chunk * 64 * NT, act,
                    [&](int m) { return (long)(from_tokens ? order[p0 + m] / top : p0 + m) * K; },
                    [&](int m) { return (long)(p0 + m) * N; });
 }
@@ -134,11 +158,14 @@ extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, cons
   PA_REQUIRE(act == 0 || act == 1, "moe_linear_mfma: unknown activation code %d", act);
   const bool few = entries <= 4 * kGmRows;
   const int cols = few ? 128 : 256;
-  dim3 grid((entries + kGmRows - 1) / kGmRows + experts, (N + cols - 1) / cols);
+  const int col_chunks = (N + cols - 1) / cols;
+  const long items = (long)((entries + kGmRows - 1) / kGmRows + experts) * col_chunks;
+  PA_REQUIRE(items <= 0x7fffff00L, "moe_linear_mfma: %ld work items exceed the grid", items);
+  dim3 grid((unsigned)(((items + 7) / 8) * 8));
   hipStream_t st = (hipStream_t)stream;
 #define PA_GM(TY, NT)                                                                                                       \
   hipLaunchKernelGGL((moe_linear_mfma_kernel<TY, NT>), grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (TY*)y, offsets, \
-                     order, experts, top, K, N, from_tokens, act)
+                     order, entries, experts, top, K, N, col_chunks, from_tokens, act)
   if (y_dtype == kBF16) {
     if (few) PA_GM(bf16, 2); else PA_GM(bf16, 4);
   } else if (y_dtype == kF32) {

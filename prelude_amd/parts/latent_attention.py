@@ -9,8 +9,8 @@ move to the query side:
     score_h(i, j) = ((W_uk[h]^T q_h^unrot(i)) . c(j)  +  q_h^rot(i) . k^rot(j)) * scale
     out_h(i)      = W_uv[h] * sum_j p_h(i, j) c(j),     p = softmax over {scores, sink_h}
 
-The sink is a number per head that joins the denominator as exp(sink_h): it has no key and no value and is not
-scaled.  Rotation pairs dimension 2i with 2i + 1 over the first ``rotary_dim`` rotated dimensions.  Scores,
+A head's sink is a learned scalar s_h: its softmax divides by sum_j exp(score_j) + exp(s_h).  Nothing is attended
+to through it (it adds to the denominator only), and the score scale does not apply to it.  Rotation pairs dimension 2i with 2i + 1 over the first ``rotary_dim`` rotated dimensions.  Scores,
 softmax, norms and angles are 32-bit whatever the engine's type.
 """
 from __future__ import annotations

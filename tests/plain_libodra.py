@@ -147,6 +147,14 @@ def tiny_config_q():
     return config(300, 128, [(a, dense(256, 2.5)), (a, moe(4, 1, 64, 64)), (a, dense(256, 2.5))], eps=1e-6)
 
 
+def tiny_config_r():
+    """Sizes that fit no 16-byte piece: a width of 100, one and two heads, a latent of 20, all experts for every
+    token, layers that differ in every size."""
+    a = mixer_cfg(1, 10, 6, 12, 20, 12, base=77.0, rot_dims=2, scale=0.4)
+    b = mixer_cfg(2, 6, 4, 10, 28, 20, base=5000.0)
+    return config(50, 100, [(a, dense(50, 1.1)), (b, moe(3, 3, 30, 18)), (b, None), (a, moe(2, 1, 14))], eps=1e-4)
+
+
 def tensor_shapes(cfg):
     V, W = cfg["vocab"], cfg["width"]
     out = {"embed": (V, W), "final.norm": (W,), "head": (V, W)}

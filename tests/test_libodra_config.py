@@ -17,7 +17,7 @@ def build(raw):
     return CausalLM(a.build_spec(a.parse_config(raw)))
 
 
-@pytest.mark.parametrize("make", [pl.tiny_config_p, pl.tiny_config_q])
+@pytest.mark.parametrize("make", [pl.tiny_config_p, pl.tiny_config_q, pl.tiny_config_r])
 def test_the_model_asks_for_the_tensors_the_design_names(make):
     raw = make()
     m = build(raw)

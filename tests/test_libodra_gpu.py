@@ -286,7 +286,8 @@ def test_experts_by_table(gpu, dtype, E, top, T, ff):
 
 
 # ---- the engine -------------------------------------------------------------------------------------------------
-CONFIGS = {"p": (pl.tiny_config_p, 11, 8), "q": (pl.tiny_config_q, 12, 16)}     # (configuration, seed, page size)
+# (configuration, seed, page size)
+CONFIGS = {"p": (pl.tiny_config_p, 11, 8), "q": (pl.tiny_config_q, 12, 16), "r": (pl.tiny_config_r, 13, 4)}
 
 
 @functools.lru_cache(maxsize=None)
@@ -317,7 +318,7 @@ def runner(name, dtype, max_tokens, **kw):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["p", "q"])
+@pytest.mark.parametrize("name", ["p", "q", "r"])
 def test_whole_prompt_every_position(gpu, name, dtype):
     toks, ref = plain_logits(name, 0, 150)
     r = runner(name, dtype, 256)
@@ -327,7 +328,7 @@ def test_whole_prompt_every_position(gpu, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["p", "q"])
+@pytest.mark.parametrize("name", ["p", "q", "r"])
 def test_prefill_then_token_by_token(gpu, name, dtype):
     toks, ref = plain_logits(name, 1, 140)
     r = runner(name, dtype, 256)
@@ -339,7 +340,7 @@ def test_prefill_then_token_by_token(gpu, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["p", "q"])
+@pytest.mark.parametrize("name", ["p", "q", "r"])
 def test_from_the_first_token_one_by_one(gpu, name, dtype):
     toks, ref = plain_logits(name, 2, 40)
     r = runner(name, dtype, 64)
@@ -348,7 +349,7 @@ def test_from_the_first_token_one_by_one(gpu, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["p", "q"])
+@pytest.mark.parametrize("name", ["p", "q", "r"])
 def test_portions_of_changing_size(gpu, name, dtype):
     toks, ref = plain_logits(name, 3, 170)
     sizes = [7, 2, 13, 2, 1, 31, 2, 9, 16, 3, 8, 2, 64, 5]
@@ -363,7 +364,7 @@ def test_portions_of_changing_size(gpu, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["p", "q"])
+@pytest.mark.parametrize("name", ["p", "q", "r"])
 def test_unequal_requests_in_one_batch_and_pages_used_again(gpu, name, dtype):
     """Six requests of unequal length through a pool that holds three of them: portions of some beside single
     tokens of others, a request ends as soon as it is fed and its pages go to the next."""
