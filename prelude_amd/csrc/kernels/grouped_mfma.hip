@@ -43,21 +43,28 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[j][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // The operands of the step after this one are asked for before this step's products, into a second set of
-  // registers: a step's loads take far longer than its products, and this keeps two steps' worth in flight.
-  bf16x8 wf[2][NT], xf[2][4];
+  // The operands of the three steps after this one are on their way while this step is multiplied, in four sets of
+  // registers named by constants (the loop takes four steps a turn): with few rows a workgroup is one chain of steps
+  // through its slice of the weight, a step's loads take some ten times as long as its products, and what streams
+  // the weight at the memory's rate is how much of it is in flight.
+  bf16x8 wf[4][NT], xf[4][4];
+  const int last_k0 = ((K - 1) / 32) * 32;
   auto load_step = [&](int k0, int b) {
+    k0 = k0 <= last_k0 ? k0 : last_k0;                           // (past the end: the last step once more, not multiplied)
     const bool kok = k0 + 8 * g + 8 <= K;
     const int kc = kok ? k0 : K - 8 - 8 * g;                    // (K is a multiple of 8: the clamped piece lies inside the row)
 #pragma unroll
     for (int j = 0; j < NT; ++j) wf[b][j] = *reinterpret_cast<const bf16x8*>(wr[j] + kc);
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
-      const bf16x8 v = *reinterpret_cast<const bf16x8*>(xr[mt < row_tiles ? mt : 0] + kc);
-      xf[b][mt] = kok ? v : bf16x8{};
+      if (mt < row_tiles) {                                      // (the same in every lane of the workgroup)
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(xr[mt] + kc);
+        xf[b][mt] = kok ? v : bf16x8{};
+      }
     }
   };
-  auto multiply = [&](int b) {
+  auto multiply = [&](int k0, int b) {
+    if (k0 >= K) return;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       if (mt < row_tiles) {
@@ -66,15 +73,18 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
       }
     }
   };
-  const int last_k0 = ((K - 1) / 32) * 32;
   load_step(0, 0);
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    load_step(k0 + 32 <= last_k0 ? k0 + 32 : last_k0, 1);      // (past the end: the last step once more, not multiplied)
-    multiply(0);
-    if (k0 + 32 < K) {
-      load_step(k0 + 64 <= last_k0 ? k0 + 64 : last_k0, 0);
-      multiply(1);
-    }
+  load_step(32, 1);
+  load_step(64, 2);
+  for (int k0 = 0; k0 < K; k0 += 128) {
+    load_step(k0 + 96, 3);
+    multiply(k0, 0);
+    load_step(k0 + 128, 0);
+    multiply(k0 + 32, 1);
+    load_step(k0 + 160, 1);
+    multiply(k0 + 64, 2);
+    load_step(k0 + 192, 2);
+    multiply(k0 + 96, 3);
   }
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
@@ -98,6 +108,43 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
   }
 }
 
+// Which expert a tile belongs to: an expert with c entries has ceil(c / rows) tiles, the tiles of all experts are
+// numbered in order.  Every lane takes an expert (64 at a time), the tiles are summed across the wavefront, and the
+// first expert whose running total passes `tile` is the one: no chain of dependent loads over the experts.
+// Returns false for a tile beyond the last.  All lanes of a wavefront call it with the same arguments.
+__device__ __forceinline__ bool find_tile(const int* __restrict__ offsets, int experts, int rows, int tile, int& e_out,
+                                          int& p0, int& p1) {
+  const int lane = threadIdx.x % kWave;
+  int before = 0;                                              // tiles of the experts of earlier rounds
+  for (int base = 0; base < experts; base += kWave) {
+    const int e = base + lane;
+    int a = 0, b = 0;
+    if (e < experts) {
+      a = offsets[e];
+      b = offsets[e + 1];
+    }
+    const int mine = (b - a + rows - 1) / rows;
+    int incl = mine;                                           // inclusive running total over the lanes
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int up = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += up;
+    }
+    const unsigned long long hit = __ballot(before + incl > tile);
+    if (hit) {
+      const int src = __ffsll((long long)hit) - 1;
+      const int first = tile - (before + __shfl(incl, src, kWave) - __shfl(mine, src, kWave));   // tile within its expert
+      const int ea = __shfl(a, src, kWave), eb = __shfl(b, src, kWave);
+      e_out = base + src;
+      p0 = ea + first * rows;
+      p1 = p0 + rows < eb ? p0 + rows : eb;
+      return true;
+    }
+    before += __shfl(incl, kWave - 1, kWave);
+  }
+  return false;
+}
+
 // Experts: blockIdx.x walks the tiles of 64 positions of all experts in order (an expert with c entries has
 // ceil(c / 64) tiles; blocks beyond the last leave).  `from_tokens`: position p reads row order[p] / top of x.
 template <typename TY, int NT>
@@ -114,22 +161,142 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __rest
   const int per_xcd = (total + 7) / 8;
   const int item = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
   if (blockIdx.x / 8 >= (unsigned)per_xcd || item >= total) return;
-  int tile = item % tiles_max, e = 0, p0 = 0, p1 = 0;
+  int e = 0, p0 = 0, p1 = 0;
   const int col_chunk = item / tiles_max;
-  for (; e < experts; ++e) {
-    const int a = offsets[e], b = offsets[e + 1];
-    const int tiles = (b - a + kGmRows - 1) / kGmRows;
-    if (tile < tiles) {
-      p0 = a + tile * kGmRows;
-      p1 = p0 + kGmRows < b ? p0 + kGmRows : b;
-      break;
-    }
-    tile -= tiles;
-  }
-  if (e >= experts) return;
+  if (!find_tile(offsets, experts, kGmRows, item % tiles_max, e, p0, p1)) return;
   grouped_tile<TY, NT>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, col_chunk * 64 * NT, act,
                    [&](int m) { return (long)(from_tokens ? order[p0 + m] / top : p0 + m) * K; },
                    [&](int m) { return (long)(p0 + m) * N; });
+}
+
+// The experts' product for many rows: a workgroup owns 128 positions of one expert and 128 outputs.  What limits
+// the kernel above at many rows is the bytes that travel from the L2 to the compute units (every wavefront loads
+// the rows of x for itself): here the 128 rows of x go through LDS once per workgroup (16-byte pieces, held in
+// registers while the step before is multiplied, two buffers, rows padded to 80 bytes), the weight still straight
+// from memory, a step ahead: 16 KB a step of k for the same products as the 32 KB above.
+constexpr int kGbRows = 128;
+constexpr int kGbStride = 40;   // elements of an LDS row: 32 of a step and 8 of padding
+
+template <typename TY>
+__global__ __launch_bounds__(256) void moe_linear_mfma_big_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
+                                                                 TY* __restrict__ y, const int* __restrict__ offsets,
+                                                                 const int* __restrict__ order, int entries, int experts,
+                                                                 int top, int K, int N, int col_chunks, int from_tokens,
+                                                                 int act) {
+  __shared__ __attribute__((aligned(16))) bf16 xs[2][kGbRows * kGbStride];
+  const int tiles_max = (entries + kGbRows - 1) / kGbRows + experts;
+  const int total = tiles_max * col_chunks;
+  const int per_xcd = (total + 7) / 8;
+  const int item = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+  if (blockIdx.x / 8 >= (unsigned)per_xcd || item >= total) return;
+  int e = 0, p0 = 0, p1 = 0;
+  const int col_chunk = item / tiles_max;
+  if (!find_tile(offsets, experts, kGbRows, item % tiles_max, e, p0, p1)) return;
+  const int n_rows = p1 - p0;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int row_tiles = (n_rows + 15) / 16;
+  const bf16* we = w + (size_t)e * N * K;
+  constexpr int NT = 2;                                        // 32 outputs a wavefront: registers for three workgroups a compute unit
+  const int nb = col_chunk * 64 * NT + wave * 16 * NT;                  // (a wavefront whose outputs do not exist still stages x)
+  const bool cols_ok = nb < N;
+  const bf16* wr[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = nb + 16 * j + r;
+    wr[j] = we + (size_t)(n < N ? n : N - 1) * K + 8 * g;
+  }
+  // this thread's two pieces of a step's x tile: piece c = thread + 256 i is row c / 4, elements 8 (c % 4)...
+  const bf16* xsrc[2];
+  int xdst[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    const int m = c / 4 < n_rows ? c / 4 : 0;
+    const long row = from_tokens ? order[p0 + m] / top : p0 + m;
+    xsrc[i] = x + row * K + 8 * (c % 4);
+    xdst[i] = (c / 4) * kGbStride + 8 * (c % 4);
+  }
+  f32x4 acc[NT][8];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) acc[j][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 wf[2][NT], xreg[2];
+  auto load_step = [&](int k0, int b) {                        // unconditional, clamped; a piece past the end of k is zeroed in x
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int kc = k0 + 8 * g + 8 <= K ? k0 : K - 8 - 8 * g;
+      wf[b][j] = *reinterpret_cast<const bf16x8*>(wr[j] + kc);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int piece = (threadIdx.x + 256 * i) % 4;
+      const bool kok = k0 + 8 * piece + 8 <= K;
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(xsrc[i] + (kok ? k0 : K - 8 - 8 * piece));
+      xreg[i] = kok ? v : bf16x8{};
+    }
+  };
+  auto stage = [&](int b) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<bf16x8*>(&xs[b][xdst[i]]) = xreg[i];
+  };
+  // (the two sets of registers and the two buffers are named by constants, the loop taking two steps a turn: an
+  // index that is only known at run time would send the register arrays to memory)
+  auto multiply = [&](int b) {
+    if (!cols_ok) return;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      bf16x8 xf[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xf[q] = *reinterpret_cast<const bf16x8*>(&xs[b][((4 * half + q) * 16 + r) * kGbStride + 8 * g]);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (4 * half + q < row_tiles) {
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+            acc[j][4 * half + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[b][j], xf[q], acc[j][4 * half + q], 0, 0, 0);
+        }
+      }
+    }
+  };
+  load_step(0, 0);
+  stage(0);
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    // step k0 from set 0 while step k0 + 32 arrives in set 1, then the other way round
+    const bool more1 = k0 + 32 < K;
+    if (more1) load_step(k0 + 32, 1);
+    multiply(0);
+    if (more1) stage(1);                                       // (everyone left that buffer at the barrier before this step)
+    __syncthreads();
+    if (!more1) break;
+    const bool more0 = k0 + 64 < K;
+    if (more0) load_step(k0 + 64, 0);
+    multiply(1);
+    if (more0) stage(0);
+    __syncthreads();
+  }
+  if (!cols_ok) return;
+#pragma unroll
+  for (int mt = 0; mt < 8; ++mt) {
+    if (mt * 16 + r >= n_rows) continue;
+    TY* yr = y + (size_t)(p0 + mt * 16 + r) * N;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = nb + 16 * j + 4 * g + i;
+        if (n < N) {
+          float v = acc[j][mt][i];
+          if (act == 1) {
+            v = fmaxf(v, 0.f);
+            v = v * v;
+          }
+          yr[n] = from_f32<TY>(v);
+        }
+      }
+  }
 }
 
 // Heads: grid (tiles of 64 tokens, heads, chunks of 64 NT outputs).
@@ -157,19 +324,34 @@ extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, cons
              entries, experts, K, N);
   PA_REQUIRE(act == 0 || act == 1, "moe_linear_mfma: unknown activation code %d", act);
   const bool few = entries <= 4 * kGmRows;
-  const int cols = few ? 128 : 256;
+  const int cols = 128;
   const int col_chunks = (N + cols - 1) / cols;
+  hipStream_t st = (hipStream_t)stream;
+  if (!few) {
+    // many rows: tiles of 128 positions with the rows of x through LDS
+    const long items = (long)((entries + kGbRows - 1) / kGbRows + experts) * col_chunks;
+    PA_REQUIRE(items <= 0x7fffff00L, "moe_linear_mfma: %ld work items exceed the grid", items);
+    dim3 grid((unsigned)(((items + 7) / 8) * 8));
+    if (y_dtype == kBF16)
+      hipLaunchKernelGGL(moe_linear_mfma_big_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (bf16*)y, offsets,
+                         order, entries, experts, top, K, N, col_chunks, from_tokens, act);
+    else if (y_dtype == kF32)
+      hipLaunchKernelGGL(moe_linear_mfma_big_kernel<float>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (float*)y, offsets,
+                         order, entries, experts, top, K, N, col_chunks, from_tokens, act);
+    else
+      return pa::fail("moe_linear_mfma: unknown output type code %d", y_dtype);
+    return check_launch("moe_linear_mfma");
+  }
   const long items = (long)((entries + kGmRows - 1) / kGmRows + experts) * col_chunks;
   PA_REQUIRE(items <= 0x7fffff00L, "moe_linear_mfma: %ld work items exceed the grid", items);
   dim3 grid((unsigned)(((items + 7) / 8) * 8));
-  hipStream_t st = (hipStream_t)stream;
 #define PA_GM(TY, NT)                                                                                                       \
   hipLaunchKernelGGL((moe_linear_mfma_kernel<TY, NT>), grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (TY*)y, offsets, \
                      order, entries, experts, top, K, N, col_chunks, from_tokens, act)
   if (y_dtype == kBF16) {
-    if (few) PA_GM(bf16, 2); else PA_GM(bf16, 4);
+    PA_GM(bf16, 2);
   } else if (y_dtype == kF32) {
-    if (few) PA_GM(float, 2); else PA_GM(float, 4);
+    PA_GM(float, 2);
   } else {
     return pa::fail("moe_linear_mfma: unknown output type code %d", y_dtype);
   }
