@@ -29,6 +29,15 @@ constexpr int kLmRows = 64;      // query rows a workgroup
 constexpr int kLmKeys = 32;      // keys a block
 constexpr int kLmPad = 8;        // elements of padding behind an LDS row
 
+// 64 pieces of 16 bytes from memory straight into LDS: lane l's piece lands at `lds_base` + 16 l.  Written as the
+// instruction itself: through the compiler's own builtin every later read of LDS first waited for all such loads
+// (it cannot tell the two buffers apart), which put the staging in line with the products instead of behind them.
+// The kernel waits for them itself (vmcnt 0) before the barrier that publishes a buffer.
+__device__ __forceinline__ void load_to_lds_16(const void* src, void* lds_base) {
+  const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(src) : "memory");
+}
+
 __device__ __forceinline__ f32x4 mfma16l(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
@@ -137,8 +146,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
       const int j = kk >> 3;
       const size_t row = (j == 0 ? row0[0] : (j == 1 ? row0[1] : (j == 2 ? row0[2] : row0[3]))) + (kk & 7);
       const bf16* src = cache + row * dk + 8 * (ch < ch_last ? ch : ch_last);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(buf + (size_t)sI * 512), 16, 0, 0);
+      load_to_lds_16(src, buf + (size_t)sI * 512);
       key += k_step_key;
       ch += k_step_ch;
       if (ch >= k_pieces) {
@@ -154,8 +162,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
       j = (j < 4 && 8 * j <= rel_last) ? j : 0;
       const size_t r0 = j == 0 ? run0[0] : (j == 1 ? run0[1] : (j == 2 ? run0[2] : run0[3]));
       const bf16* src = cache_t + r0 + (size_t)vrow * page_size;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(buf + (size_t)(k_loads + sI) * 512), 16, 0, 0);
+      load_to_lds_16(src, buf + (size_t)(k_loads + sI) * 512);
     }
   };
 
