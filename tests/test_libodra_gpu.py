@@ -431,3 +431,24 @@ def test_greedy_generation_through_the_scheduler(gpu):
         for _ in range(12):
             seq.append(int(pl.forward(cfg, w, seq)[-1].argmax()))
         assert out.token_ids == seq[len(p):], f"prompt of {len(p)}"
+
+
+def test_command_line_with_the_pools_sized_from_free_memory(gpu, capsys):
+    """``python -m prelude_amd`` on a Libodra folder, nothing given but the model: the pools take what the device has
+    left after a measured step, steps are replayed from graphs, and the greedy tokens are the same as with weights
+    drawn again from the folder's own values in 32-bit."""
+    from prelude_amd import cli
+    name = "q"
+    path, cfg, w = folder(name)
+    prompt = plain_logits(name, 40, 11)[0]
+    assert cli.main(["--model", path, "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "6", "--temperature", "0"]) == 0
+    rec = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert rec["finish_reason"] == "length" and len(rec["token_ids"]) == 6
+    # bfloat16 may part from the plain greedy path where two logits are close; the first token's margin is checked instead
+    ref = pl.forward(cfg, w, prompt)[-1]
+    top2 = torch.topk(ref, 2).values
+    if float(top2[0] - top2[1]) > 0.2 * float(ref.std()):
+        assert rec["token_ids"][0] == int(ref.argmax())
+    assert cli.main(["--model", path, "--random-weights", "--prompt-len", "5", "--max-tokens", "3", "--max-cache-tokens", "256"]) == 0
+    rec = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert len(rec["token_ids"]) == 3 and all(0 <= t < cfg["vocab"] for t in rec["token_ids"])
