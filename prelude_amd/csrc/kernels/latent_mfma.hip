@@ -121,51 +121,68 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   const int buf_elems = (k_loads + v_loads) * 512;             // 64 pieces of 8 elements a load
   const int ch_last = dk / 8 - 1;
   // Where this lane's piece of each load lies does not change from block to block: piece i = 64 * load + lane of
-  // the rows is key i / k_pieces, piece i % k_pieces; the loads of a wavefront are 256 pieces apart, so the pair is
-  // stepped, not divided, and the divisions happen once.
-  const int k_step_key = 256 / k_pieces, k_step_ch = 256 % k_pieces;
-  const int k_key0 = (wave * 64 + lane) / k_pieces, k_ch0 = (wave * 64 + lane) % k_pieces;
+  // the rows is key i / k_pieces, piece i % k_pieces; of the transposed copy element i / 5, run i % 5 of 8 keys (the
+  // fifth is padding).  So each load's share of the address is worked out once, before the first block: the offset
+  // inside the block's run of 8 keys (24 bits) and which of the block's four runs it is (the bits above).  A block
+  // then costs a load a choice among four bases and an addition.  (Pages hold multiples of 8 keys, so a run lies in
+  // one page.  Pieces of padding, elements and keys that do not exist take the place of ones that do.)
+  constexpr int KS = ((kLmKeys * (QS * 4 + 1) + 63) / 64 + 3) / 4;      // loads of rows a wavefront, at most
+  constexpr int VS = ((RT * 16 * 5 + 63) / 64 + 3) / 4;                 // loads of the copy a wavefront, at most
+  unsigned kinfo[KS], vinfo[VS];
+#pragma unroll
+  for (int sl = 0; sl < KS; ++sl) {
+    const int i = (wave + 4 * sl) * 64 + lane;
+    int key = i / k_pieces, ch = i % k_pieces;
+    key = key < kLmKeys ? key : kLmKeys - 1;
+    ch = ch < ch_last ? ch : ch_last;
+    kinfo[sl] = (unsigned)((key & 7) * dk + 8 * ch) | ((unsigned)(key >> 3) << 24);
+  }
+#pragma unroll
+  for (int sl = 0; sl < VS; ++sl) {
+    const int i = (wave + 4 * sl) * 64 + lane;
+    int vrow = i / 5, j = i % 5;
+    vrow = vrow < rank ? vrow : rank - 1;
+    j = j < 4 ? j : 0;
+    vinfo[sl] = (unsigned)(vrow * page_size) | ((unsigned)j << 24);
+  }
   auto issue_block = [&](int b0, bf16* buf) {
     const int last = end_wg - 1;
     const int rel_last = last - b0;                              // >= 0: the block holds a key of the range
-    // the pages of the block's four runs of 8 keys (pages hold multiples of 8 keys) and the runs' places in them
-    size_t row0[4], run0[4];                                     // first row of a run in the cache; the run in the copy
+    // where the block's four runs of 8 keys start, in the cache and in the copy (the same for every lane); a run past
+    // the range takes the place of the last one inside it
+    const bf16* krun[4];
+    const bf16* vrun[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int kc = 8 * j <= rel_last ? b0 + 8 * j : (last & ~7);
       const int at = kc / page_size;
       const int page = table[at];
       const size_t pg = page >= 0 ? page : 0, place = kc - at * page_size;
-      row0[j] = pg * page_size + place;
-      run0[j] = pg * rank * page_size + place;
+      krun[j] = cache + (pg * page_size + place) * dk;
+      vrun[j] = cache_t + pg * rank * page_size + place;
     }
-    int key = k_key0, ch = k_ch0;
-    for (int sI = wave; sI < k_loads; sI += 4) {
-      int kk = key < kLmKeys ? key : kLmKeys - 1;
-      kk = kk < rel_last ? kk : rel_last;
-      const int j = kk >> 3;
-      const size_t row = (j == 0 ? row0[0] : (j == 1 ? row0[1] : (j == 2 ? row0[2] : row0[3]))) + (kk & 7);
-      const bf16* src = cache + row * dk + 8 * (ch < ch_last ? ch : ch_last);
-      load_to_lds_16(src, buf + (size_t)sI * 512);
-      key += k_step_key;
-      ch += k_step_ch;
-      if (ch >= k_pieces) {
-        ch -= k_pieces;
-        ++key;
+#pragma unroll
+    for (int sl = 0; sl < KS; ++sl) {
+      const int sI = wave + 4 * sl;
+      if (sI < k_loads) {
+        const unsigned j = kinfo[sl] >> 24;
+        const bf16* base = j == 0 ? krun[0] : (j == 1 ? krun[1] : (j == 2 ? krun[2] : krun[3]));
+        load_to_lds_16(base + (kinfo[sl] & 0xffffffu), buf + (size_t)sI * 512);
       }
     }
-    // the transposed copy: piece i is element i / 5, run i % 5 (the fifth is padding)
-    for (int sI = wave; sI < v_loads; sI += 4) {
-      const int i = sI * 64 + lane;
-      int vrow = i / 5, j = i % 5;
-      vrow = vrow < rank ? vrow : rank - 1;
-      j = (j < 4 && 8 * j <= rel_last) ? j : 0;
-      const size_t r0 = j == 0 ? run0[0] : (j == 1 ? run0[1] : (j == 2 ? run0[2] : run0[3]));
-      const bf16* src = cache_t + r0 + (size_t)vrow * page_size;
-      load_to_lds_16(src, buf + (size_t)(k_loads + sI) * 512);
+#pragma unroll
+    for (int sl = 0; sl < VS; ++sl) {
+      const int sI = wave + 4 * sl;
+      if (sI < v_loads) {
+        const unsigned j = vinfo[sl] >> 24;
+        const bf16* base = j == 0 ? vrun[0] : (j == 1 ? vrun[1] : (j == 2 ? vrun[2] : vrun[3]));
+        load_to_lds_16(base + (vinfo[sl] & 0xffffffu), buf + (size_t)(k_loads + sI) * 512);
+      }
     }
   };
 
+  const int wave_pos_min = __shfl(pos, 0, kWave);              // the wavefront's rows ascend: its first row sees least,
+  const int wave_lo_max = __shfl(lo_row, 15, kWave);           // its last row's window starts last
   bf16* const buf0 = reinterpret_cast<bf16*>(lds_raw);
   if (lo_wg < end_wg) issue_block(lo_wg, buf0);
   int it = 0;
@@ -207,28 +224,41 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
       }
     }
     // ---- mask, running maximum, probabilities ----
+    // (a block that every row of the wavefront sees whole, which is most of them, skips the mask)
     float bm = -INFINITY;
+    if (b0 + kLmKeys - 1 <= wave_pos_min && b0 >= wave_lo_max && b0 + kLmKeys <= end_wg) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int kidx = b0 + 8 * g + 4 * t + i;
-        const bool ok = kidx <= pos && kidx >= lo_row && kidx < end_wg;
-        s[t][i] = ok ? s[t][i] : -INFINITY;
-        bm = fmaxf(bm, s[t][i]);
-      }
+        for (int i = 0; i < 4; ++i) bm = fmaxf(bm, s[t][i]);
+    } else {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kidx = b0 + 8 * g + 4 * t + i;
+          const bool ok = kidx <= pos && kidx >= lo_row && kidx < end_wg;
+          s[t][i] = ok ? s[t][i] : -INFINITY;
+          bm = fmaxf(bm, s[t][i]);
+        }
+    }
     bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
     bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
-    const float m_new = fmaxf(m, bm);
+    // The exponentials are taken against a reference that follows the running maximum lazily: it moves, and the
+    // sums are rescaled, only when a score exceeds it by 2^8 (then probabilities stay below 256, which 32-bit sums
+    // and bfloat16 operands hold as well as values below 1); after the first blocks that is rare.
+    const bool move = m == -INFINITY || (bm - m) * c > 8.f;
+    const float m_new = move ? bm : m;
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f((m - m_use) * c);
+    const float shift = -m_use * c;
+    const float alpha = move ? __builtin_amdgcn_exp2f(fmaf(m, c, shift)) : 1.0f;
     float psum = 0.f;
     bf16x8 pf;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = exp2f((s[t][i] - m_use) * c);       // exp2(-inf) = 0 for masked keys
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[t][i], c, shift));       // 2^-inf = 0 for masked keys
         psum += p;
         pf[4 * t + i] = (bf16)p;
       }
@@ -388,6 +418,7 @@ using namespace pa;
 // Sizes the matrix-core kernel takes: 16-byte rows, at most 512 + 64 elements, pages of a multiple of 8 keys.
 extern "C" int pa_latent_attn_mfma_supports(int rank, int rot, int page_size) {
   return rank > 0 && rot >= 0 && rank % 8 == 0 && rot % 8 == 0 && rank <= 512 && rot <= 64 && page_size > 0 && page_size % 8 == 0 &&
+         page_size <= 16384 &&   // (an element's offset in the transposed copy, rank * page_size, is kept in 24 bits)
          latent_mfma_lds(rank, rot) <= 160 * 1024;
 }
 
