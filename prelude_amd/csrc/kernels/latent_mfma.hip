@@ -210,9 +210,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
         bf16x8 ka[kBatch], kb[kBatch];
 #pragma unroll
         for (int j = 0; j < kBatch; ++j) {
-          const int ks = k0 + j < QS ? k0 + j : QS - 1;      // (a step past the latent's own reads inside the buffer and is not used)
-          ka[j] = *reinterpret_cast<const bf16x8*>(kr0 + 32 * (ks < dk_steps ? ks : 0));
-          kb[j] = *reinterpret_cast<const bf16x8*>(kr1 + 32 * (ks < dk_steps ? ks : 0));
+          // (offsets known when compiled: a step past the latent's own width reads on into the buffer -- the rows
+          // are followed by the transposed copy, so it stays inside -- and is not multiplied)
+          const int ks = k0 + j < QS ? k0 + j : QS - 1;
+          ka[j] = *reinterpret_cast<const bf16x8*>(kr0 + 32 * ks);
+          kb[j] = *reinterpret_cast<const bf16x8*>(kr1 + 32 * ks);
         }
 #pragma unroll
         for (int j = 0; j < kBatch; ++j) {
