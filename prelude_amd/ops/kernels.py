@@ -1271,10 +1271,12 @@ LATENT_MAX_WIDTH = 1024   # rank + rot of a cached latent vector the attention k
 
 
 # Keys a split of the matrix-core kernel, for steps of single tokens: a workgroup walks its split block by block, one
-# after the other, so the shortest split that still leaves the launch within LATENT_SPLIT_WORKGROUPS workgroups is the
-# fastest (8 sequences of 4,096 keys: 512 workgroups of 2 blocks instead of 128 of 8)
+# after the other, and a compute unit holds one workgroup, so the shortest split that still leaves the launch within
+# one round of the chip (LATENT_SPLIT_WORKGROUPS workgroups) is the fastest: 8 sequences of 4,096 keys take 41.6 us in
+# 256 workgroups of 4 blocks, 52.6 in 512 of 2 (two rounds) and 82 in 128 of 8; 32 sequences 115 us at 256 keys a
+# split and 136 at 128
 LATENT_SPLIT_KEYS = (64, 128, 256)
-LATENT_SPLIT_WORKGROUPS = 768
+LATENT_SPLIT_WORKGROUPS = 256
 LATENT_MAX_SPLITS = 4096     # what the merge kernel takes; contexts beyond 4,096 splits of 256 keys get longer splits
 
 
