@@ -78,7 +78,7 @@ _KERNEL_API = {
     "pa_latent_attn": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
     "pa_latent_attn_mfma_supports": (I, [I, I, I]),
     "pa_latent_attn_mfma_workspace": (c_long, [I, I, I, I]),
-    "pa_latent_attn_mfma": (I, [P, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I]),
+    "pa_latent_attn_mfma": (I, [P, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I]),
     "pa_moe_choices_by_table": (I, [P, P, P, P, I, I, I, I]),
     "pa_moe_order": (I, [P, P, I, I, P, P, P, P]),
     "pa_moe_linear": (I, [P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I]),

@@ -189,13 +189,14 @@ int pa_latent_attn(void* stream, int dtype, const void* q, const void* cache, co
                    int rot, int page_size, int window, float scale);
 // The same on the matrix cores (latent_mfma.hip; bfloat16): the sequences seq_ids[0..n_seqs) (null: 0..n_seqs) with
 // cu_q[s+1] - cu_q[s] tokens each (at most max_q_len) ending at context_lens[s].  n_splits > 1, for sequences of one
-// token: keys in splits of split_keys, partials in ws (pa_latent_attn_mfma_workspace 32-bit words), merged in split order.
+// token: keys in splits of split_keys, partials in ws (pa_latent_attn_mfma_workspace 32-bit words), merged in split order;
+// wave_splits: a split is a wavefront that reads the cache directly (many sequences) instead of a workgroup that stages it.
 int pa_latent_attn_mfma_supports(int rank, int rot, int page_size);
 long pa_latent_attn_mfma_workspace(int n_seqs, int nh, int rank, int n_splits);
 int pa_latent_attn_mfma(void* stream, const void* q, const void* cache, const void* cache_t, const float* sink, const int* block_table,
                         int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, void* ws,
                         int n_seqs, int max_q_len, int nh, int rank, int rot, int page_size, int window, float scale,
-                        int split_keys, int n_splits);
+                        int split_keys, int n_splits, int wave_splits);
 
 // ---- experts (moe.hip) ----
 int pa_moe_choices_by_table(void* stream, const int* ids, const int* table, int* choice, int tokens, int top, int vocab,

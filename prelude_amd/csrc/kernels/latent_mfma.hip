@@ -339,6 +339,170 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     }
 }
 
+// Steps of single tokens: a sequence brings only `heads` rows, one tile of 16 for 16 heads, so staging a block in LDS
+// for four wavefronts serves one of them, and a workgroup walking its blocks one after the other is bound by the
+// latency of each.  Here a wavefront is a split of its own: it takes 16 heads of one sequence and its own range of
+// keys, reads both operands straight from the cache in 16-byte pieces (a row of a key for the scores; eight keys of an
+// element from the transposed copy for the weighted sum: what the cache's two layouts are for), batches of loads in
+// flight, no LDS and no barrier; four such wavefronts a workgroup keep four blocks of a compute unit's memory
+// traffic in flight.  Every wavefront leaves a partial for the merge kernel.
+// Grid (sequences, ceil(splits / 4), tiles of 16 heads); split z = 4 blockIdx.y + wavefront.
+template <int RT, int QS>
+__global__ __launch_bounds__(256) void latent_attn_decode_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ cache, const bf16* __restrict__ cache_t,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, float* __restrict__ ws, int nh, int rank, int rot,
+    int page_size, int window, float scale, int split_keys, int n_splits) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int g = lane / 16, r = lane % 16;
+  const int z = blockIdx.y * 4 + wave;
+  if (z >= n_splits) return;
+  const int seq = seq_ids ? seq_ids[blockIdx.x] : blockIdx.x;
+  const int tok = cu_q[seq];
+  const int pos = context_lens[seq] - 1;
+  const int dk = rank + rot;
+  const int dk_steps = (dk + 31) / 32;
+  const int v_tiles = (rank + 15) / 16;
+  const int* table = block_table + (size_t)seq * table_stride;
+  const int head0 = blockIdx.z * 16;
+  const int head = head0 + r < nh ? head0 + r : nh - 1;
+  const bool row_ok = head0 + r < nh;
+  const int lo_row = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int lo = z * split_keys, end = lo + split_keys;
+  lo = lo > lo_row ? lo : lo_row;
+  end = end < pos + 1 ? end : pos + 1;
+  const int b_first = (lo / kLmKeys) * kLmKeys;
+
+  bf16x8 qf[QS];
+  {
+    const bf16* qr = q + ((size_t)tok * nh + head) * dk;
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+      const int d = 32 * s + 8 * g;
+      bf16x8 v = {};
+      if (d + 8 <= dk) v = *reinterpret_cast<const bf16x8*>(qr + d);
+      qf[s] = v;
+    }
+  }
+  f32x4 o[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const float c = scale * kLog2eL;
+  const int last = end - 1;
+
+  for (int b0 = b_first; b0 < end; b0 += kLmKeys) {
+    // this lane's two key rows (tile t: key 8 (r / 4) + 4 t + r % 4) and its run of 8 keys in the copy, clamped into
+    // the range (what a clamped key brings is masked)
+    const bf16* kr[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      int kidx = b0 + 8 * (r / 4) + 4 * t + (r % 4);
+      kidx = kidx < last ? kidx : last;
+      const int at = kidx / page_size;
+      const int page = table[at];
+      kr[t] = cache + ((size_t)(page >= 0 ? page : 0) * page_size + (kidx - at * page_size)) * dk + 8 * g;
+    }
+    const bf16* vr;
+    {
+      int kidx = b0 + 8 * g;
+      kidx = kidx < (last & ~7) ? kidx : (last & ~7);
+      const int at = kidx / page_size;
+      const int page = table[at];
+      vr = cache_t + ((size_t)(page >= 0 ? page : 0) * rank + r) * page_size + (kidx - at * page_size);
+    }
+    f32x4 s[2];
+    s[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int kBatch = 6;
+#pragma unroll
+    for (int k0 = 0; k0 < QS; k0 += kBatch) {
+      bf16x8 ka[kBatch], kb[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        int ks = k0 + j < QS ? k0 + j : QS - 1;
+        ks = ks < dk_steps ? ks : dk_steps - 1;
+        const int d = 32 * ks + 8 * g + 8 <= dk ? 32 * ks : dk - 8 - 8 * g;      // (a piece past the row's end: the last one; q is zero there)
+        ka[j] = *reinterpret_cast<const bf16x8*>(kr[0] + d);
+        kb[j] = *reinterpret_cast<const bf16x8*>(kr[1] + d);
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        if (k0 + j < QS && k0 + j < dk_steps) {
+          s[0] = mfma16l(ka[j], qf[k0 + j], s[0]);
+          s[1] = mfma16l(kb[j], qf[k0 + j], s[1]);
+        }
+      }
+    }
+    float bm = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int kidx = b0 + 8 * g + 4 * t + i;
+        const bool ok = kidx >= lo && kidx < end;
+        s[t][i] = ok ? s[t][i] : -INFINITY;
+        bm = fmaxf(bm, s[t][i]);
+      }
+    bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
+    bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
+    const bool move = m == -INFINITY || (bm - m) * c > 8.f;
+    const float m_new = move ? bm : m;
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float shift = -m_use * c;
+    const float alpha = move ? __builtin_amdgcn_exp2f(fmaf(m, c, shift)) : 1.0f;
+    float psum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[t][i], c, shift));
+        psum += p;
+        pf[4 * t + i] = (bf16)p;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    const bool rescale = __any(alpha != 1.0f);
+    constexpr int vBatch = 8;
+#pragma unroll
+    for (int t0 = 0; t0 < RT; t0 += vBatch) {
+      if (t0 < v_tiles) {
+        bf16x8 vf[vBatch];
+#pragma unroll
+        for (int j = 0; j < vBatch; ++j) {
+          int e = 16 * (t0 + j) + r;                           // this lane's element of tile t0 + j, clamped into the latent
+          e = e < rank ? e : rank - 1;
+          vf[j] = *reinterpret_cast<const bf16x8*>(vr + (size_t)(e - r) * page_size);
+        }
+#pragma unroll
+        for (int j = 0; j < vBatch; ++j) {
+          if (t0 + j < RT && t0 + j < v_tiles) {
+            if (rescale) o[t0 + j] *= alpha;
+            o[t0 + j] = mfma16l(vf[j], pf, o[t0 + j]);
+          }
+        }
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (!row_ok) return;
+  float* w = ws + (((size_t)blockIdx.x * nh + head) * n_splits + z) * (rank + 2);
+  if (g == 0) {
+    w[0] = m * scale;
+    w[1] = l;
+  }
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+    if (t < v_tiles)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = 16 * t + 4 * g + i;
+        if (d < rank) w[2 + d] = o[t][i];
+      }
+}
+
 // out[row] = sum over the splits' partials, each scaled by exp(its maximum - the largest), then the sink.
 // One workgroup a row; the splits' factors are worked out once (in LDS), then every thread adds its elements over
 // the splits in order, eight loads in flight.
@@ -432,11 +596,12 @@ extern "C" long pa_latent_attn_mfma_workspace(int n_seqs, int nh, int rank, int 
 // q [tokens, heads, rank + rot], cache [pages, page, rank + rot] and its latents transposed, cache_t [pages, rank, page]
 // -> out [tokens, heads, rank] for the sequences seq_ids[0..n_seqs) (null: sequences
 // 0..n_seqs), each with cu_q[s+1] - cu_q[s] tokens ending at context_lens[s]; max_q_len bounds their tokens.
-// n_splits > 1 (sequences of one token only): the keys in splits of split_keys, partials in ws, merged here.
+// n_splits > 1 (sequences of one token only): the keys in splits of split_keys, partials in ws, merged here; a split is
+// a workgroup of the staged kernel, or with `wave_splits` a wavefront of the kernel that reads the cache directly.
 extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cache, const void* cache_t, const float* sink, const int* block_table,
                                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                                    void* ws, int n_seqs, int max_q_len, int nh, int rank, int rot, int page_size,
-                                   int window, float scale, int split_keys, int n_splits) {
+                                   int window, float scale, int split_keys, int n_splits, int wave_splits) {
   if (n_seqs == 0) return 0;
   PA_REQUIRE(pa_latent_attn_mfma_supports(rank, rot, page_size), "latent_attn_mfma: a latent of %d + %d is not a size it takes", rank, rot);
   PA_REQUIRE(n_seqs > 0 && max_q_len > 0 && nh > 0 && table_stride > 0 && window >= 0,
@@ -446,11 +611,31 @@ extern "C" int pa_latent_attn_mfma(void* stream, const void* q, const void* cach
   PA_REQUIRE(n_splits <= kMergeMaxSplits, "latent_attn_mfma: %d splits are more than the %d the merge takes", n_splits, kMergeMaxSplits);
   PA_REQUIRE(n_splits >= 1 && (n_splits == 1 || (split_keys > 0 && split_keys % kLmKeys == 0 && ws && max_q_len == 1)),
              "latent_attn_mfma: %d splits of %d keys need a workspace, whole blocks and sequences of one token", n_splits, split_keys);
+  hipStream_t st = (hipStream_t)stream;
+  if (n_splits > 1 && wave_splits) {
+    // sequences of one token, many of them: a wavefront a split, operands straight from the cache, then the merge
+    const int head_tiles = (nh + 15) / 16;
+    PA_REQUIRE(n_seqs <= 0x7fffffff && head_tiles <= 65535, "latent_attn_mfma: %d sequences or %d heads exceed the grid", n_seqs, nh);
+    dim3 grid(n_seqs, (n_splits + 3) / 4, head_tiles);
+#define PA_LD(RT, QS)                                                                                                    \
+  hipLaunchKernelGGL((latent_attn_decode_kernel<RT, QS>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)cache,     \
+                     (const bf16*)cache_t, block_table, table_stride, seq_ids, cu_q, context_lens, (float*)ws, nh, rank, rot, \
+                     page_size, window, scale, split_keys, n_splits)
+    if (rank <= 64) PA_LD(4, 4);
+    else if (rank <= 128) PA_LD(8, 6);
+    else if (rank <= 256) PA_LD(16, 10);
+    else PA_LD(32, 18);
+#undef PA_LD
+    if (int e = check_launch("latent_attn_decode")) return e;
+    hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(n_seqs * nh), dim3(rank >= 256 ? 256 : 64), 0, st, (const float*)ws, sink,
+                       seq_ids, cu_q, (bf16*)out, nh, rank, n_splits);
+    return check_launch("latent_attn_merge");
+  }
   const long tiles = ((long)max_q_len * nh + kLmRows - 1) / kLmRows;
-  PA_REQUIRE(tiles <= 0x7fffffffL && n_seqs <= 65535 && n_splits <= 65535, "latent_attn_mfma: the grid %ld x %d x %d is too large", tiles, n_seqs, n_splits);
+  PA_REQUIRE(tiles <= 0x7fffffffL && n_seqs <= 65535 && n_splits <= 65535, "latent_attn_mfma: the grid %ld x %d x %d is too large", tiles,
+             n_seqs, n_splits);
   dim3 grid((unsigned)tiles, n_seqs, n_splits);
   const size_t lds = latent_mfma_lds(rank, rot);
-  hipStream_t st = (hipStream_t)stream;
   int rc;
 #define PA_LM(RT, QS)                                                                                                  \
   rc = launch_latent_mfma<RT, QS>(st, grid, lds, (const bf16*)q, (const bf16*)cache, (const bf16*)cache_t, sink, block_table, table_stride,  \

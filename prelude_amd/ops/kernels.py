@@ -1270,24 +1270,38 @@ def moe_combine(y: torch.Tensor, eo: ExpertOrder, weight: float, base: Optional[
 LATENT_MAX_WIDTH = 1024   # rank + rot of a cached latent vector the attention kernels take
 
 
-# Keys a split of the matrix-core kernel, for steps of single tokens: a workgroup walks its split block by block, one
-# after the other, and a compute unit holds one workgroup, so the shortest split that still leaves the launch within
-# one round of the chip (LATENT_SPLIT_WORKGROUPS workgroups) is the fastest: 8 sequences of 4,096 keys take 41.6 us in
-# 256 workgroups of 4 blocks, 52.6 in 512 of 2 (two rounds) and 82 in 128 of 8; 32 sequences 115 us at 256 keys a
-# split and 136 at 128
+# Keys a split, for steps of single tokens.  Two kernels take them.  Few sequences (fewer than LATENT_WAVE_SPLITS_FROM
+# tiles of 16 heads): a split is a workgroup of the staged kernel, whose loads of a block all go out at once (8
+# sequences of 4,096 keys: 41.6 us against 54 the other way).  Many: a split is a wavefront that reads the cache
+# directly, four a workgroup (32 sequences: 95 us against 115; 64: 167 against 224; 8 of 32,768 keys: 171 against 234;
+# one of 32,768 keys in 1,024 splits of a block each: 130 us, which is why a single sequence stays with the staged kernel).
+# Either way a workgroup walks its keys block by block and a compute unit holds one workgroup, so the shortest split
+# that still leaves the launch within one round of the chip (LATENT_SPLIT_WORKGROUPS workgroups) is the fastest.
 LATENT_SPLIT_KEYS = (64, 128, 256)
+LATENT_WAVE_SPLIT_KEYS = (32, 64, 128, 256)
 LATENT_SPLIT_WORKGROUPS = 256
+LATENT_WAVE_SPLITS_FROM = 24      # ... or where the staged kernel's longest splits no longer fit one round
 LATENT_MAX_SPLITS = 4096     # what the merge kernel takes; contexts beyond 4,096 splits of 256 keys get longer splits
 
 
-def latent_split_keys(n_seqs: int, max_context: int) -> int:
-    for keys in LATENT_SPLIT_KEYS:
-        if n_seqs * -(-int(max_context) // keys) <= LATENT_SPLIT_WORKGROUPS:
-            return keys
+def latent_split_plan(n_seqs: int, max_context: int, heads: int = 16):
+    """(keys a split, whether a split is a wavefront) for a step of ``n_seqs`` single tokens."""
+    head_tiles = -(-int(heads) // 16)
+    per_wave = (n_seqs * head_tiles >= LATENT_WAVE_SPLITS_FROM
+                or n_seqs * -(-int(max_context) // LATENT_SPLIT_KEYS[-1]) > LATENT_SPLIT_WORKGROUPS)
+    for keys in (LATENT_WAVE_SPLIT_KEYS if per_wave else LATENT_SPLIT_KEYS):
+        splits = -(-int(max_context) // keys)
+        groups = n_seqs * head_tiles * -(-splits // 4) if per_wave else n_seqs * splits
+        if splits <= LATENT_MAX_SPLITS and groups <= LATENT_SPLIT_WORKGROUPS:
+            return keys, per_wave
     keys = LATENT_SPLIT_KEYS[-1]
     while -(-int(max_context) // keys) > LATENT_MAX_SPLITS:
         keys *= 2
-    return keys
+    return keys, per_wave
+
+
+def latent_split_keys(n_seqs: int, max_context: int, heads: int = 16) -> int:
+    return latent_split_plan(n_seqs, max_context, heads)[0]
 
 
 def latent_attention_mfma_supported(rank: int, rot: int, page_size: int) -> bool:
@@ -1297,10 +1311,11 @@ def latent_attention_mfma_supported(rank: int, rot: int, page_size: int) -> bool
 def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, cache_t: torch.Tensor, sink: Optional[torch.Tensor], block_table: torch.Tensor,
                           seq_ids: Optional[torch.Tensor], n_seqs: int, cu_q: torch.Tensor, context_lens: torch.Tensor,
                           out: torch.Tensor, max_q_len: int, rank: int, window: int, scale: float,
-                          max_context: int = 0) -> None:
+                          max_context: int = 0, per_wave: Optional[bool] = None) -> None:
     """The matrix-core kernel for the sequences ``seq_ids`` (None: all ``n_seqs`` of the step); writes their rows of
     ``out`` [T, heads, rank].  ``max_context`` > 0 with ``max_q_len`` 1 cuts the keys into splits of
-    ``latent_split_keys`` keys whose partials a second kernel merges: what fills the chip when every sequence feeds one token."""
+    ``latent_split_plan`` keys whose partials a second kernel merges: what fills the chip when every sequence feeds one
+    token.  ``per_wave`` (tests and measurements) fixes which of the two kernels takes the splits."""
     _dev(q, cache, cache_t, sink, block_table, seq_ids, cu_q, context_lens, out)
     _f32(sink, "sink")
     t, nh, dk = q.shape
@@ -1312,14 +1327,15 @@ def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, cache_t: torch.T
     if n_seqs == 0:
         return
     splits, ws = 1, None
-    split_keys = latent_split_keys(n_seqs, max_context)
+    split_keys, planned = latent_split_plan(n_seqs, max_context, nh)
+    per_wave = planned if per_wave is None else bool(per_wave)
     if max_q_len == 1 and max_context > split_keys:
         splits = -(-int(max_context) // split_keys)
         ws = torch.empty(int(kernels().pa_latent_attn_mfma_workspace(n_seqs, nh, rank, splits)), dtype=torch.float32, device=q.device)
     check(kernels().pa_latent_attn_mfma(_stream(), _ptr(q), _ptr(cache), _ptr(cache_t), _ptr(sink), _ptr(block_table), block_table.shape[1],
                                         _ptr(seq_ids), _ptr(cu_q), _ptr(context_lens), _ptr(out), _ptr(ws), int(n_seqs),
                                         int(max_q_len), nh, int(rank), dk - int(rank), cache.shape[1], int(window), float(scale),
-                                        split_keys, splits))
+                                        split_keys, splits, 1 if per_wave else 0))
 
 
 def latent_attention(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], group, step, rank: int,

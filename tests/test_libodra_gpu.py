@@ -227,10 +227,20 @@ def test_latent_attention_on_the_matrix_cores(gpu, H, rank, rot, page):
     cu1 = torch.arange(5, dtype=torch.int32, device=gpu)
     out = torch.zeros((4, H, rank), dtype=torch.bfloat16, device=gpu)
     for window in (0, 290):
-        K.latent_attention_mfma(torch.cat(ql).to(gpu), cache, cache_t, sink.to(gpu), table, None, 4, cu1, cl, out, 1, rank, window, scale,
-                                max_context=768)
         want = torch.cat([_plain_latent_attention(ql[i], lat[i], sink, rank, scale, torch.tensor([ctx[i] - 1]), window) for i in range(4)])
-        close(out, want, dtype, f"single tokens in splits, window {window}", scale=1.0)
+        for per_wave in (False, True):      # a split a workgroup that stages its keys; a split a wavefront that reads the cache
+            out.zero_()
+            K.latent_attention_mfma(torch.cat(ql).to(gpu), cache, cache_t, sink.to(gpu), table, None, 4, cu1, cl, out, 1, rank, window,
+                                    scale, max_context=768, per_wave=per_wave)
+            close(out, want, dtype, f"single tokens in splits, window {window}, per wavefront {per_wave}", scale=1.0)
+    # a chosen list of sequences, the other rows left alone, both ways
+    for per_wave in (False, True):
+        out.zero_()
+        K.latent_attention_mfma(torch.cat(ql).to(gpu), cache, cache_t, sink.to(gpu), table, torch.tensor([2, 0], dtype=torch.int32, device=gpu),
+                                2, cu1, cl, out, 1, rank, 0, scale, max_context=768, per_wave=per_wave)
+        want = torch.cat([_plain_latent_attention(ql[i], lat[i], sink, rank, scale, torch.tensor([ctx[i] - 1]), 0) for i in (0, 2)])
+        close(out[[0, 2]], want, dtype, f"chosen sequences, per wavefront {per_wave}", scale=1.0)
+        assert float(out[[1, 3]].abs().max()) == 0.0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
