@@ -287,3 +287,159 @@ class LibodraConfig:
         norm = _obj(raw, "norm", a)
         return cls(vocab=_positive(raw, "vocab", int, a, ""), width=_positive(raw, "width", int, a, ""),
                    norm_eps=_positive(norm, "eps", float, a, "norm."), layers=tuple(layers))
+
+
+# ---------------------------------------------------------------------------
+@dataclasses.dataclass(frozen=True)
+class LightningMixerConfig:
+    heads: int
+    dim: int                    # query/key dimensions a head
+    vdim: int                   # value dimensions a head
+    decay: Tuple[float, ...]    # one a head
+
+
+@dataclasses.dataclass(frozen=True)
+class LongWaveScaling:
+    factor: float
+    low: float
+    high: float
+    original: int
+
+
+@dataclasses.dataclass(frozen=True)
+class SinkAttentionConfig:
+    heads: int
+    kv_heads: int
+    dim: int                    # query/key dimensions a head; the values are the keys, so also the value's
+    scale: float
+    rot_base: float
+    rot_dims: int               # how many of a head's first dimensions turn
+    rot_scaling: Optional[LongWaveScaling]
+
+
+@dataclasses.dataclass(frozen=True)
+class FazopelMlpConfig:
+    kind: str                   # "dense" | "moe"
+    ff: int = 0                 # dense: inner size; moe: an expert's inner size
+    limit: float = 0.0          # moe: an expert's clamp
+    experts: int = 0
+    top: int = 0
+    route_scale: float = 1.0
+    shared_ff: int = 0          # moe: inner size of the shared expert, 0 = none
+    shared_limit: float = 0.0
+
+
+@dataclasses.dataclass(frozen=True)
+class FazopelLayerConfig:
+    type: str                   # "lightning" | "attention"
+    mixer: object               # LightningMixerConfig | SinkAttentionConfig
+    mlp: Optional[FazopelMlpConfig]
+    weights_of: Optional[int]   # the layer whose tensors this one uses (its own cache or state); None: its own
+
+
+@dataclasses.dataclass(frozen=True)
+class FazopelConfig:
+    """Fazopel: a decoder whose layers are listed one by one in ``layers``; a layer norms each branch's output before
+    adding it.  Its mixer is linear attention with a decaying state (``lightning``) or grouped-query attention whose
+    values are its keys and whose softmax has an empty sink (``attention``); its feed-forward is dense (squared relu),
+    a mixture of routed experts with an optional shared one, or absent.  A layer may use another layer's tensors
+    (``weights_of``).  Every size and constant is read from here; there is no longest position and no
+    end-of-sequence id."""
+    vocab: int
+    width: int
+    norm_eps: float
+    layers: Tuple[FazopelLayerConfig, ...]
+
+    ARCH = "Fazopel"
+    MIXERS = ("lightning", "attention")
+
+    @classmethod
+    def _mixer(cls, kind: str, m: Mapping[str, Any], mw: str):
+        a = cls.ARCH
+        heads = _positive(m, "heads", int, a, mw)
+        dim = _positive(m, "dim", int, a, mw)
+        vdim = _positive(m, "vdim", int, a, mw)
+        if kind == "lightning":
+            decay = m.get("decay")
+            if not isinstance(decay, list) or len(decay) != heads or \
+                    not all(isinstance(x, (int, float)) and not isinstance(x, bool) and 0.0 <= x <= 1.0 for x in decay):
+                raise ConfigError(f"failed to parse {a} config: `{mw}decay` must list one number in [0, 1] for each of "
+                                  f"the {heads} heads, got {decay!r}")
+            return LightningMixerConfig(heads, dim, vdim, tuple(float(x) for x in decay))
+        kv_heads = _positive(m, "kv_heads", int, a, mw)
+        if heads % kv_heads:
+            raise ConfigError(f"failed to parse {a} config: `{mw}heads` ({heads}) is no multiple of `kv_heads` ({kv_heads})")
+        if vdim != dim:
+            raise ConfigError(f"failed to parse {a} config: `{mw}vdim` ({vdim}) must equal `dim` ({dim}): the values are the keys")
+        rot = _obj(m, "rot", a, mw)
+        rw = mw + "rot."
+        dims = _get(rot, "dims", int, a)
+        if dims % 2 or dims > dim:
+            raise ConfigError(f"failed to parse {a} config: `{rw}dims` ({dims}) must be even and at most `dim` ({dim})")
+        sc = _obj(rot, "scaling", a, rw, optional=True)
+        scaling = None
+        if sc is not None:
+            sw = rw + "scaling."
+            scaling = LongWaveScaling(_positive(sc, "factor", float, a, sw), _positive(sc, "low", float, a, sw),
+                                      _positive(sc, "high", float, a, sw), _positive(sc, "original", int, a, sw))
+            if not scaling.high > scaling.low:
+                raise ConfigError(f"failed to parse {a} config: `{sw}high` ({scaling.high}) must exceed `low` ({scaling.low})")
+        return SinkAttentionConfig(heads, kv_heads, dim, _positive(m, "scale", float, a, mw),
+                                   _positive(rot, "base", float, a, rw), dims, scaling)
+
+    @classmethod
+    def _mlp(cls, f: Optional[Mapping[str, Any]], fw: str) -> Optional[FazopelMlpConfig]:
+        a = cls.ARCH
+        if f is None:
+            return None
+        fk = _get(f, "kind", str, a)
+        if fk == "dense":
+            return FazopelMlpConfig("dense", ff=_positive(f, "ff", int, a, fw))
+        if fk != "moe":
+            raise ConfigError(f"failed to parse {a} config: `{fw}kind` {fk!r} is not one of ['dense', 'moe']")
+        router = _obj(f, "router", a, fw)
+        expert = _obj(f, "expert", a, fw)
+        shared = _obj(f, "shared", a, fw, optional=True)
+        mlp = FazopelMlpConfig(
+            "moe", ff=_positive(expert, "ff", int, a, fw + "expert."), limit=_positive(expert, "limit", float, a, fw + "expert."),
+            experts=_positive(router, "experts", int, a, fw + "router."), top=_positive(router, "top", int, a, fw + "router."),
+            route_scale=_positive(router, "scale", float, a, fw + "router."),
+            shared_ff=_positive(shared, "ff", int, a, fw + "shared.") if shared is not None else 0,
+            shared_limit=_positive(shared, "limit", float, a, fw + "shared.") if shared is not None else 0.0)
+        if mlp.top > mlp.experts:
+            raise ConfigError(f"failed to parse {a} config: `{fw}router.top` ({mlp.top}) exceeds `router.experts` ({mlp.experts})")
+        return mlp
+
+    @classmethod
+    def from_dict(cls, raw: Mapping[str, Any]) -> "FazopelConfig":
+        a = cls.ARCH
+        layers_raw = raw.get("layers")
+        if not isinstance(layers_raw, list) or not layers_raw:
+            raise ConfigError(f"failed to parse {a} config: `layers` must be a non-empty list")
+        layers = []
+        for i, lr in enumerate(layers_raw):
+            w = f"layers[{i}]."
+            if not isinstance(lr, dict):
+                raise ConfigError(f"failed to parse {a} config: `layers[{i}]` must be an object")
+            kind = _get(lr, "type", str, a)
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"failed to parse {a} config: `{w}type` {kind!r} is not one of {list(cls.MIXERS)}")
+            src = _get(lr, "weights_of", int, a, default=None)
+            layer = FazopelLayerConfig(kind, cls._mixer(kind, _obj(lr, "mixer", a, w), w + "mixer."),
+                                       cls._mlp(_obj(lr, "mlp", a, w, optional=True), w + "mlp."), src)
+            if src is not None:
+                if not 0 <= src < len(layers_raw) or src == i:
+                    raise ConfigError(f"failed to parse {a} config: `{w}weights_of` ({src}) names no other layer")
+            layers.append(layer)
+        for i, layer in enumerate(layers):
+            if layer.weights_of is not None:
+                j = layer.weights_of
+                if layers[j].weights_of is not None:
+                    raise ConfigError(f"failed to parse {a} config: `layers[{i}].weights_of` names layer {j}, which has no "
+                                      f"tensors of its own")
+                if dataclasses.replace(layers[j], weights_of=None) != dataclasses.replace(layer, weights_of=None):
+                    raise ConfigError(f"failed to parse {a} config: `layers[{i}]` uses the tensors of layer {j} but "
+                                      f"differs from it")
+        norm = _obj(raw, "norm", a)
+        return cls(vocab=_positive(raw, "vocab", int, a, ""), width=_positive(raw, "width", int, a, ""),
+                   norm_eps=_positive(norm, "eps", float, a, "norm."), layers=tuple(layers))

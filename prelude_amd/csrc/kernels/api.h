@@ -47,6 +47,14 @@ int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_w
                       void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int hd, int rot,
                       int page_size, float eps);
 
+// pa_qknorm_rope_kv from the rotary frequencies alone (inv_freq [rot / 2], the angle position * inv_freq[j] taken in
+// 32-bit in the kernel: no tables, no longest position); v_from_k: qkv is [tokens, (nh + nkv) * hd] and the cached
+// value of a head is its key as projected, before norm and rotation.
+int pa_qknorm_rope_kv_freq(void* stream, int dtype, const void* qkv, const float* q_weight, const float* k_weight,
+                           const float* inv_freq, const int* positions, const int* slots, void* q_out, void* k_cache,
+                           void* v_cache, int tokens, int nh, int nkv, int hd, int rot, int page_size, float eps,
+                           int v_from_k);
+
 // C[m, n] = X[m, k] W[n, k]^T, bfloat16 with 32-bit accumulation, by hipBLASLt called directly; `workspace` is
 // device memory its kernels may use.  The first call with a shape makes and keeps that shape's plan in host memory.
 int pa_gemm_library(void* stream, const void* x, const void* w, void* c, int m, int n, int k, long ldx, long ldc,
@@ -95,6 +103,13 @@ int pa_pack_tiles(void* stream, const void* w, void* out, int n, int k);
 int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
                     const int* block_table, int table_stride, const int* seq_of_token, const int* positions, void* out,
                     int tokens, int nh, int nkv, int hd, int page_size, int window, float scale, float softcap);
+
+// pa_attn_generic with a sink per head (sink [nh], 32-bit, in the units of the scaled scores): the softmax divides
+// by sum_j exp(s_j) + exp(sink_h).
+int pa_attn_generic_sink(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
+                         const int* block_table, int table_stride, const int* seq_of_token, const int* positions, void* out,
+                         int tokens, int nh, int nkv, int hd, int page_size, int window, float scale, float softcap,
+                         const float* sink);
 
 // Matrix-core attention in bfloat16 (K cache [page, nkv, page_size, hd], V cache [page, nkv, hd, page_size]).
 // seq_ids lists the sequences of the step a call handles; cu_q[s] is the first packed token row of sequence s,
@@ -168,6 +183,23 @@ int pa_clamped_gate(void* stream, int dtype, const void* gate_up, void* out, int
 // out = max(x, 0)^2
 int pa_relu_squared(void* stream, int dtype, const void* x, void* out, long total);
 
+// residual (32-bit) += y * rsqrt(mean(y^2) + eps) * w, y = x (of `dtype`) or `slices` partial sums; copy (or null,
+// of `dtype`) receives the new residual rounded: a branch's output normed and added to the stream.
+int pa_rmsnorm_branch(void* stream, int dtype, const void* x, const float* parts, int slices, long slice_stride,
+                      float* residual, const float* w, void* copy, int nrows, int hidden, float eps);
+// out[t, i] = o[t, i] * rsqrt(mean(o[t]^2) + eps) * w[i] * sigmoid(gate[t, i]); o 32-bit, gate and out of `dtype`,
+// gate rows gate_stride elements apart.
+int pa_gated_rmsnorm(void* stream, int dtype, const float* o, const void* gate, long gate_stride, const float* w, void* out,
+                     int nrows, int width, float eps);
+
+// ---- linear attention with a decaying state (lightning.hip) ----
+// S_t = decay[h] S_(t-1) + k_t v_t^T, out[t, h, :] = S_t^T q_t; q, k [heads, dim] and v [heads, vdim] of token t at
+// qkv[t * ld + q_off / k_off / v_off ..] of `dtype`, passed through act (0 none, 1 SiLU); state [slots, heads, dim,
+// vdim] 32-bit; sequence s owns rows cu_q[s] .. cu_q[s + 1] and slot state_slots[s]; out [tokens, heads, vdim] 32-bit.
+int pa_lightning_attn(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off, const float* decay,
+                      float* state, const int* state_slots, const int* cu_q, float* out, int nseq, int tokens, int heads,
+                      int dim, int vdim, int act);
+
 // ---- attention through a latent (latent.hip) ----
 // in [tokens, q_rank + rank + rot]: cq_out [tokens, q_rank] = RMSNorm(first part) * wq; into the cache row slots[t]
 // ([rank + rot] elements a token): RMSNorm(second part) * wc, then the third part with its first rot_dims elements
@@ -205,8 +237,15 @@ int pa_moe_order(void* stream, const int* choice, int entries, int experts, int*
 int pa_moe_linear(void* stream, int x_dtype, int w_dtype, int y_dtype, const void* x, const void* wt, void* y,
                   const int* offsets, const int* order, int entries, int experts, int top, int K, int N, int from_tokens,
                   int act);
+// out[t] = (base_scale ? base_scale[t] : 1) * base[t] + sum_j w[t, j] * y[place[t * top + j]]
 int pa_moe_combine(void* stream, int dtype, const float* y, const int* place, const float* weights, float weight,
-                   const void* base, void* out, int tokens, int top, int width);
+                   const void* base, const float* base_scale, void* out, int tokens, int top, int width);
+// A router: logits [tokens, ld] (32-bit; the first `experts` columns), s = softmax(logits); the `top` experts with the
+// largest s + correction[e] (correction null: none) -> choice [tokens, top]; weights [tokens, top] = their s over the
+// sum of the chosen s (+ 1e-20), times scale.  gate_out (or null) [tokens] = sigmoid(logits[t, gate_col]), a gate a
+// token for a shared expert, from one more column of the same product.
+int pa_moe_route(void* stream, const float* logits, int ld, const float* correction, int* choice, float* weights,
+                 float* gate_out, int tokens, int experts, int top, float scale, int gate_col);
 // The same two products on the matrix cores (grouped_mfma.hip; bfloat16 operands, K a multiple of 8): the weight as
 // stored, [group, N, K].
 int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, const void* w, void* y, const int* offsets, const int* order,

@@ -30,7 +30,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, T* __restrict__ out, int nh, int nkv, int hd, int page_size, int window,
-    float scale, float softcap) {
+    float scale, float softcap, const float* __restrict__ sink) {
   __shared__ float qs[kAttnWaves][kAttnMaxHd];
   __shared__ float ps[kAttnWaves][kWave];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -92,7 +92,12 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
   }
   if (active) {
     T* orow = out + ((size_t)t * nh + h) * hd;
-    const float inv = 1.0f / l;
+    float inv = 1.0f / l;
+    if (sink) {   // one more term exp(sink) of the denominator that brings no value
+      const float m_fin = fmaxf(m, sink[h]);
+      const float alpha = expf(m - m_fin);
+      inv = alpha / (l * alpha + expf(sink[h] - m_fin));
+    }
 #pragma unroll
     for (int e = 0; e < kAttnMaxHd / kWave; ++e) {
       const int d = lane + e * kWave;
@@ -105,10 +110,10 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
 
 using namespace pa;
 
-extern "C" int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
+static int attn_generic_launch(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
                                const int* block_table, int table_stride, const int* seq_of_token,
                                const int* positions, void* out, int tokens, int nh, int nkv, int hd, int page_size,
-                               int window, float scale, float softcap) {
+                               int window, float scale, float softcap, const float* sink) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && nh > 0 && nkv > 0 && page_size > 0 && table_stride > 0,
              "attn_generic: bad sizes tokens=%d nh=%d nkv=%d page=%d table_stride=%d", tokens, nh, nkv, page_size,
@@ -122,13 +127,31 @@ extern "C" int pa_attn_generic(void* stream, int dtype, const void* q, const voi
   if (dtype == kF32) {
     hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kAttnWaves * kWave), 0, st, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, block_table, table_stride, seq_of_token, positions,
-                       (float*)out, nh, nkv, hd, page_size, window, scale, softcap);
+                       (float*)out, nh, nkv, hd, page_size, window, scale, softcap, sink);
   } else if (dtype == kBF16) {
     hipLaunchKernelGGL(attn_generic_kernel<bf16>, grid, dim3(kAttnWaves * kWave), 0, st, (const bf16*)q,
                        (const bf16*)k_cache, (const bf16*)v_cache, block_table, table_stride, seq_of_token, positions,
-                       (bf16*)out, nh, nkv, hd, page_size, window, scale, softcap);
+                       (bf16*)out, nh, nkv, hd, page_size, window, scale, softcap, sink);
   } else {
     return pa::fail("attn_generic: unknown element type code %d", dtype);
   }
   return check_launch("attn_generic");
+}
+
+extern "C" int pa_attn_generic(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
+                               const int* block_table, int table_stride, const int* seq_of_token,
+                               const int* positions, void* out, int tokens, int nh, int nkv, int hd, int page_size,
+                               int window, float scale, float softcap) {
+  return attn_generic_launch(stream, dtype, q, k_cache, v_cache, block_table, table_stride, seq_of_token, positions, out, tokens,
+                             nh, nkv, hd, page_size, window, scale, softcap, nullptr);
+}
+
+// The same with a sink per head (sink [nh], 32-bit, in the units of the scaled scores): the softmax divides by
+// sum_j exp(s_j) + exp(sink_h); nothing is attended to through it.
+extern "C" int pa_attn_generic_sink(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
+                                    const int* block_table, int table_stride, const int* seq_of_token,
+                                    const int* positions, void* out, int tokens, int nh, int nkv, int hd, int page_size,
+                                    int window, float scale, float softcap, const float* sink) {
+  return attn_generic_launch(stream, dtype, q, k_cache, v_cache, block_table, table_stride, seq_of_token, positions, out, tokens,
+                             nh, nkv, hd, page_size, window, scale, softcap, sink);
 }

@@ -7,10 +7,12 @@
 // leave at once), so a captured step replays; no sum depends on what else the step holds.
 //
 //   pa_moe_choices_by_table   which experts: a row of an integer table per token id (no router)
+//   pa_moe_route              which experts: a router's scores, a correction added for the choice alone, the
+//                             chosen scores normed over their sum; beside them a gate for the shared expert
 //   pa_moe_order              entries by expert: offsets [E + 1], order [entries] (position -> entry),
 //                             place [entries] (entry -> position)
 //   pa_moe_linear             y[p, :] = act(W[expert of p] x[row of p, :]) over the ordered positions p
-//   pa_moe_combine            out[t] = base[t] + sum_j weight[t, j] * y[place[t * top + j]]
+//   pa_moe_combine            out[t] = base_scale[t] * base[t] + sum_j weight[t, j] * y[place[t * top + j]]
 #include "common.h"
 #include "api.h"
 
@@ -24,6 +26,82 @@ __global__ void moe_choices_by_table_kernel(const int* __restrict__ ids, const i
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   int x = table[(size_t)id * top + e % top];
   choice[e] = x < 0 ? 0 : (x >= experts ? experts - 1 : x);   // a table out of range must not index outside the weights
+}
+
+// One wavefront a token.  logits [tokens, ld] 32-bit: the first `experts` columns are the router's, column `gate_col`
+// (>= 0) is a gate of its own.  s = softmax(logits) over the experts; the `top` experts with the largest
+// s + correction are chosen (the lowest index among equals), in descending order of that sum; their weights are
+// s / (sum of the chosen s + 1e-20) * scale; gate_out[t] = sigmoid(logits[t, gate_col]).  A lane holds the experts
+// lane, lane + 64, ..: up to kRouteMax of them.
+constexpr int kRoutePerLane = 8;
+constexpr int kRouteMax = kRoutePerLane * kWave;
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction,
+                                                       int* __restrict__ choice, float* __restrict__ weights,
+                                                       float* __restrict__ gate_out, int tokens, int experts, int top,
+                                                       float scale, int gate_col) {
+  const int lane = threadIdx.x % kWave;
+  const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (t >= tokens) return;
+  const float* z = logits + (size_t)t * ld;
+  float s[kRoutePerLane], c[kRoutePerLane];
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < kRoutePerLane; ++j) {
+    const int e = lane + j * kWave;
+    s[j] = e < experts ? z[e] : -INFINITY;
+    m = fmaxf(m, s[j]);
+  }
+  m = wave_max(m);
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < kRoutePerLane; ++j) {
+    const int e = lane + j * kWave;
+    s[j] = e < experts ? expf(s[j] - m) : 0.f;
+    sum += s[j];
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int j = 0; j < kRoutePerLane; ++j) {
+    const int e = lane + j * kWave;
+    s[j] = s[j] / sum;
+    c[j] = e < experts ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
+  }
+  float chosen_sum = 0.f;
+  float mine = 0.f;      // lane i < top: the score of the i-th chosen expert
+  int mine_e = 0;
+  for (int i = 0; i < top; ++i) {
+    float best = -INFINITY, best_s = 0.f;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < kRoutePerLane; ++j) {
+      const int e = lane + j * kWave;
+      if (c[j] > best) best = c[j], best_e = e, best_s = s[j];   // ascending e within a lane: the lowest index among equals
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, kWave), os = __shfl_xor(best_s, off, kWave);
+      const int oe = __shfl_xor(best_e, off, kWave);
+      if (ob > best || (ob == best && oe < best_e)) best = ob, best_e = oe, best_s = os;
+    }
+#pragma unroll
+    for (int j = 0; j < kRoutePerLane; ++j)
+      if (lane + j * kWave == best_e) c[j] = -INFINITY;
+    chosen_sum += best_s;
+    if (lane == i % kWave && i < kWave) mine = best_s, mine_e = best_e;
+    if (i >= kWave && lane == 0) {   // more than 64 chosen: written one by one, weights in a second pass below
+      choice[(size_t)t * top + i] = best_e;
+      weights[(size_t)t * top + i] = best_s;
+    }
+  }
+  const float norm = scale / (chosen_sum + 1e-20f);
+  if (lane < top) {
+    choice[(size_t)t * top + lane] = mine_e;
+    weights[(size_t)t * top + lane] = mine * norm;
+  }
+  if (top > kWave && lane == 0)
+    for (int i = kWave; i < top; ++i) weights[(size_t)t * top + i] *= norm;
+  if (gate_out && lane == 0) gate_out[t] = gate_col >= 0 ? 1.0f / (1.0f + expf(-z[gate_col])) : 1.0f;
 }
 
 // One workgroup an expert.  Pass 0 (counts == out): counts[e] = entries of e.  Pass 1: the expert's start is the
@@ -139,15 +217,17 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const TX* __restrict__ 
 // same `weight` for all when it is null.
 template <typename T>
 __global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const float* __restrict__ weights,
-                                   float weight, const T* __restrict__ base, T* __restrict__ out, int top, int width) {
+                                   float weight, const T* __restrict__ base, const float* __restrict__ base_scale,
+                                   T* __restrict__ out, int top, int width) {
   const int t = blockIdx.x;
+  const float bs = base_scale ? base_scale[t] : 1.0f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float s = 0.f;
     for (int j = 0; j < top; ++j) {
       const int e = t * top + j;
       s += (weights ? weights[e] : weight) * y[(size_t)place[e] * width + i];
     }
-    if (base) s += to_f32(base[(size_t)t * width + i]);
+    if (base) s += base_scale ? bs * to_f32(base[(size_t)t * width + i]) : to_f32(base[(size_t)t * width + i]);
     out[(size_t)t * width + i] = from_f32<T>(s);
   }
 }
@@ -198,17 +278,29 @@ extern "C" int pa_moe_linear(void* stream, int x_dtype, int w_dtype, int y_dtype
   return check_launch("moe_linear");
 }
 
+extern "C" int pa_moe_route(void* stream, const float* logits, int ld, const float* correction, int* choice, float* weights,
+                            float* gate_out, int tokens, int experts, int top, float scale, int gate_col) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && experts > 0 && top > 0 && top <= experts && ld >= experts, "moe_route: bad sizes tokens=%d experts=%d top=%d ld=%d",
+             tokens, experts, top, ld);
+  PA_REQUIRE(experts <= kRouteMax, "moe_route: %d experts are more than the %d the kernel takes", experts, kRouteMax);
+  PA_REQUIRE(gate_col < ld, "moe_route: gate column %d is outside rows of %d", gate_col, ld);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + 3) / 4), dim3(256), 0, (hipStream_t)stream, logits, ld, correction, choice,
+                     weights, gate_out, tokens, experts, top, scale, gate_col);
+  return check_launch("moe_route");
+}
+
 extern "C" int pa_moe_combine(void* stream, int dtype, const float* y, const int* place, const float* weights, float weight,
-                              const void* base, void* out, int tokens, int top, int width) {
+                              const void* base, const float* base_scale, void* out, int tokens, int top, int width) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && top > 0 && width > 0, "moe_combine: bad sizes tokens=%d top=%d width=%d", tokens, top, width);
   hipStream_t st = (hipStream_t)stream;
   if (dtype == kF32)
     hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(tokens), dim3(256), 0, st, y, place, weights, weight, (const float*)base,
-                       (float*)out, top, width);
+                       base_scale, (float*)out, top, width);
   else if (dtype == kBF16)
     hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(tokens), dim3(256), 0, st, y, place, weights, weight, (const bf16*)base,
-                       (bf16*)out, top, width);
+                       base_scale, (bf16*)out, top, width);
   else
     return pa::fail("moe_combine: unknown element type code %d", dtype);
   return check_launch("moe_combine");

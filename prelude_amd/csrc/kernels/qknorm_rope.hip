@@ -27,7 +27,8 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
                                       const float* __restrict__ sin_table, const int* __restrict__ positions,
                                       const int* __restrict__ slots, T* __restrict__ q_out,
                                       T* __restrict__ k_cache, T* __restrict__ v_cache, int tokens, int nh, int nkv,
-                                      int hd, int rot, int page_size, float eps) {
+                                      int hd, int rot, int page_size, float eps, const float* __restrict__ inv_freq,
+                                      int v_from_k) {
   __shared__ float normed[kQkWaves][kMaxHeadDim];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int heads = nh + 2 * nkv;
@@ -35,7 +36,9 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
   const bool active = unit < (long long)tokens * heads;
   const int t = active ? (int)(unit / heads) : 0;
   const int h = active ? (int)(unit % heads) : 0;
-  const T* src = qkv + ((size_t)t * heads + h) * hd;
+  // values that are the keys as projected: the row holds nh + nkv heads, and a value head reads its key head
+  const int src_heads = v_from_k ? nh + nkv : heads;
+  const T* src = qkv + ((size_t)t * src_heads + ((v_from_k && h >= nh + nkv) ? h - nkv : h)) * hd;
 
   // Where this head goes.
   T* dst = nullptr;
@@ -97,20 +100,22 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
   if (!active || is_v || !dst) return;
   const int half = rot / 2;
   const int pos = rot > 0 ? positions[t] : 0;
-  const float* c = cos_table + (size_t)pos * half;
-  const float* s = sin_table + (size_t)pos * half;
+  const float* c = cos_table ? cos_table + (size_t)pos * half : nullptr;
+  const float* s = sin_table ? sin_table + (size_t)pos * half : nullptr;
 #pragma unroll
   for (int e = 0; e < kMaxHeadDim / kWave; ++e) {
     const int i = lane + e * kWave;
     if (i >= hd) continue;
     float r = x[e];
     if (rotate && i < rot) {
-      if (i < half) {
-        r = x[e] * c[i] - normed[wave][i + half] * s[i];
-      } else {
-        const int j = i - half;
-        r = normed[wave][j] * s[j] + x[e] * c[j];
+      const int j = i < half ? i : i - half;
+      float cj, sj;
+      if (c) {
+        cj = c[j], sj = s[j];
+      } else {   // no tables: the angle position * frequency and its cosine and sine, in 32-bit
+        sincosf((float)pos * inv_freq[j], &sj, &cj);
       }
+      r = i < half ? x[e] * cj - normed[wave][i + half] * sj : normed[wave][j] * sj + x[e] * cj;
     }
     dst[i] = from_f32<T>(r);
   }
@@ -299,22 +304,23 @@ __global__ __launch_bounds__(kQkWaves* kWave) void qknorm_rope_kv_wide_kernel(
 
 using namespace pa;
 
-extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_weight,
+static int qknorm_rope_kv_launch(void* stream, int dtype, const void* qkv, const float* q_weight,
                                  const float* k_weight, const float* cos_table, const float* sin_table,
                                  const int* positions, const int* slots, void* q_out, void* k_cache,
                                  void* v_cache, int tokens, int nh, int nkv, int hd, int rot, int page_size,
-                                 float eps) {
+                                 float eps, const float* inv_freq, int v_from_k) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && nh > 0 && nkv >= 0 && page_size > 0, "qknorm_rope_kv: bad sizes tokens=%d nh=%d nkv=%d page=%d",
              tokens, nh, nkv, page_size);
   PA_REQUIRE(hd > 0 && hd <= kMaxHeadDim, "qknorm_rope_kv: head_dim %d is outside 1..%d", hd, kMaxHeadDim);
   PA_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "qknorm_rope_kv: rotary width %d must be even and at most head_dim %d",
              rot, hd);
-  PA_REQUIRE(rot == 0 || (cos_table && sin_table && positions), "qknorm_rope_kv: rotary tables or positions missing");
+  PA_REQUIRE(rot == 0 || (((cos_table && sin_table) || inv_freq) && positions),
+             "qknorm_rope_kv: rotary tables (or frequencies) or positions missing");
   const long long units = (long long)tokens * (nh + 2 * nkv);
   const unsigned blocks = (unsigned)((units + kQkWaves - 1) / kQkWaves);
   hipStream_t st = (hipStream_t)stream;
-  if (rot == hd && rot > 0 && (hd == 64 || hd == 128 || hd == 256) && (dtype == kF32 || dtype == kBF16)) {
+  if (rot == hd && rot > 0 && cos_table && !v_from_k && (hd == 64 || hd == 128 || hd == 256) && (dtype == kF32 || dtype == kBF16)) {
     const int vgroup = tokens >= 64 ? 8 : 1;   // runs of eight tokens pay only in prompt portions
     const long long v_units = (long long)((tokens + vgroup - 1) / vgroup) * nkv;
     // many tokens: five loads in flight per wavefront; few: one, so that there are wavefronts enough
@@ -351,13 +357,34 @@ extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const
   if (dtype == kF32) {
     hipLaunchKernelGGL(qknorm_rope_kv_kernel<float>, dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const float*)qkv,
                        q_weight, k_weight, cos_table, sin_table, positions, slots, (float*)q_out, (float*)k_cache,
-                       (float*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps);
+                       (float*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k);
   } else if (dtype == kBF16) {
     hipLaunchKernelGGL(qknorm_rope_kv_kernel<bf16>, dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const bf16*)qkv,
                        q_weight, k_weight, cos_table, sin_table, positions, slots, (bf16*)q_out, (bf16*)k_cache,
-                       (bf16*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps);
+                       (bf16*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k);
   } else {
     return pa::fail("qknorm_rope_kv: unknown element type code %d", dtype);
   }
   return check_launch("qknorm_rope_kv");
+}
+
+extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_weight,
+                                 const float* k_weight, const float* cos_table, const float* sin_table,
+                                 const int* positions, const int* slots, void* q_out, void* k_cache,
+                                 void* v_cache, int tokens, int nh, int nkv, int hd, int rot, int page_size,
+                                 float eps) {
+  return qknorm_rope_kv_launch(stream, dtype, qkv, q_weight, k_weight, cos_table, sin_table, positions, slots, q_out, k_cache,
+                               v_cache, tokens, nh, nkv, hd, rot, page_size, eps, nullptr, 0);
+}
+
+// The same from the frequencies alone (inv_freq [rot / 2]: the angle position * inv_freq[j] and its cosine and sine are
+// taken here, in 32-bit, so there is no table and no longest position), and, with v_from_k, for a projection of
+// nh + nkv heads whose values are its keys as projected: the cached value is the key before norm and rotation.
+extern "C" int pa_qknorm_rope_kv_freq(void* stream, int dtype, const void* qkv, const float* q_weight,
+                                      const float* k_weight, const float* inv_freq, const int* positions, const int* slots,
+                                      void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int hd,
+                                      int rot, int page_size, float eps, int v_from_k) {
+  PA_REQUIRE(rot == 0 || inv_freq, "qknorm_rope_kv: rotary frequencies missing");
+  return qknorm_rope_kv_launch(stream, dtype, qkv, q_weight, k_weight, nullptr, nullptr, positions, slots, q_out, k_cache,
+                               v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k ? 1 : 0);
 }

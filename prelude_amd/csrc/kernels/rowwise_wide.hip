@@ -3,13 +3,16 @@
 //   - RMSNorm of (x + residual) with the residual kept in 32-bit, whatever the element type of x and the output;
 //   - a gated pair with both halves clamped: g = min(g, limit), u = clamp(u, -limit, limit),
 //     y = g * sigmoid(alpha * g) * (u + 1);
-//   - the square of relu.
+//   - the square of relu;
+//   - a branch's output brought to unit RMS, scaled and added to the 32-bit stream (a layer whose norm sits on the
+//     sublayer's output: x <- x + norm(f(x))), with a copy of the new stream in the engine's type for the next reader;
+//   - a row of 32-bit values brought to unit RMS, scaled, and multiplied by the sigmoid of a gate.
 #include "common.h"
 #include "api.h"
 
 namespace pa {
 
-// s = x (+ residual), all in 32-bit; residual <- s unrounded (unless `rows`); out = round(s * rsqrt(mean(s^2) + eps) * w).
+// s = x (+ residual) (or the residual's rows alone, x and parts null), all in 32-bit; residual <- s unrounded (unless `rows`); out = round(s * rsqrt(mean(s^2) + eps) * w).
 // x may come as `slices` 32-bit partial sums, [slices, rows, hidden], added in order in place of the load of x.
 // One workgroup a row; NV elements a thread held in registers between the two passes when the row fits.
 template <typename T, int NV>
@@ -30,7 +33,7 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(const T* __restrict__
       v = pr[i];
       for (int p = 1; p < slices; ++p) v += pr[(size_t)p * slice_stride + i];
     } else {
-      v = to_f32(xr[i]);
+      v = xr ? to_f32(xr[i]) : 0.f;   // neither: the norm of the residual's rows alone
     }
     if (rr) v += rr[i];
     return v;
@@ -115,6 +118,119 @@ __global__ void relu_squared_vec_kernel(const bf16* __restrict__ x, bf16* __rest
   *reinterpret_cast<bf16x8*>(out + 8 * i) = o;
 }
 
+// residual <- residual + y * rsqrt(mean(y^2) + eps) * w, all in 32-bit; copy (or null) = the new residual rounded to
+// T.  y is x, or `slices` partial sums added in order.  One workgroup a row; up to NV * 256 elements are held in
+// registers between the two passes, longer rows are read twice.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void rmsnorm_branch_kernel(const T* __restrict__ x, const float* __restrict__ parts,
+                                                            int slices, size_t slice_stride, float* __restrict__ residual,
+                                                            const float* __restrict__ w, T* __restrict__ copy, int hidden,
+                                                            float eps) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const T* xr = x ? x + r * hidden : nullptr;
+  const float* pr = parts ? parts + r * hidden : nullptr;
+  float* rr = residual + r * hidden;
+  T* cr = copy ? copy + r * hidden : nullptr;
+  auto value = [&](int i) {
+    if (!pr) return to_f32(xr[i]);
+    float v = pr[i];
+    for (int p = 1; p < slices; ++p) v += pr[(size_t)p * slice_stride + i];
+    return v;
+  };
+  float ss = 0.f;
+  if (NV > 0) {
+    float v[NV > 0 ? NV : 1];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = threadIdx.x + j * 256;
+      v[j] = i < hidden ? value(i) : 0.f;
+      ss += v[j] * v[j];
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = threadIdx.x + j * 256;
+      if (i < hidden) {
+        const float s = rr[i] + v[j] * inv * w[i];
+        rr[i] = s;
+        if (cr) cr[i] = from_f32<T>(s);
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += 256) {
+      const float s = value(i);
+      ss += s * s;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += 256) {
+      const float s = rr[i] + value(i) * inv * w[i];
+      rr[i] = s;
+      if (cr) cr[i] = from_f32<T>(s);
+    }
+  }
+}
+
+// out[t, i] = o[t, i] * rsqrt(mean_i(o[t, :]^2) + eps) * w[i] * sigmoid(gate[t, i]); o 32-bit, gate of type T in rows
+// gate_stride elements apart (it may lie inside a wider projection).  One workgroup a row.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                           size_t gate_stride, const float* __restrict__ w,
+                                                           T* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const float* orow = o + r * width;
+  const T* grow = gate + r * gate_stride;
+  T* dst = out + r * width;
+  float ss = 0.f;
+  float v[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = threadIdx.x + j * 256;
+    v[j] = i < width ? orow[i] : 0.f;
+    ss += v[j] * v[j];
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < width) dst[i] = from_f32<T>(v[j] * inv * w[i] / (1.0f + expf(-to_f32(grow[i]))));
+  }
+}
+
+template <typename T>
+static void launch_branch(hipStream_t st, const T* x, const float* parts, int slices, size_t slice_stride, float* residual,
+                          const float* w, T* copy, int nrows, int hidden, float eps) {
+#define PA_BRANCH(NV)                                                                                                 \
+  hipLaunchKernelGGL((rmsnorm_branch_kernel<T, NV>), dim3(nrows), dim3(256), 0, st, x, parts, slices, slice_stride,  \
+                     residual, w, copy, hidden, eps)
+  if (hidden <= 256) PA_BRANCH(1);
+  else if (hidden <= 1024) PA_BRANCH(4);
+  else if (hidden <= 2048) PA_BRANCH(8);
+  else if (hidden <= 4096) PA_BRANCH(16);
+  else if (hidden <= 8192) PA_BRANCH(32);
+  else PA_BRANCH(0);
+#undef PA_BRANCH
+}
+
+template <typename T>
+static int launch_gated(hipStream_t st, const float* o, const T* gate, size_t gate_stride, const float* w, T* out, int nrows,
+                        int width, float eps) {
+#define PA_GATED(NV)                                                                                                  \
+  hipLaunchKernelGGL((gated_rmsnorm_kernel<T, NV>), dim3(nrows), dim3(256), 0, st, o, gate, gate_stride, w, out, width, eps)
+  if (width <= 256) PA_GATED(1);
+  else if (width <= 1024) PA_GATED(4);
+  else if (width <= 2048) PA_GATED(8);
+  else if (width <= 4096) PA_GATED(16);
+  else if (width <= 8192) PA_GATED(32);
+  else return pa::fail("gated_rmsnorm: rows of %d elements are more than the 8192 the kernel takes", width);
+#undef PA_GATED
+  return 0;
+}
+
 template <typename T>
 static void launch_wide(hipStream_t st, const T* x, const float* parts, int slices, size_t slice_stride, float* residual,
                         const float* w, T* out, const int* rows, int nrows, int hidden, float eps) {
@@ -139,7 +255,8 @@ extern "C" int pa_rmsnorm_wide(void* stream, int dtype, const void* x, const flo
                                float eps) {
   if (nrows == 0) return 0;
   PA_REQUIRE(nrows > 0 && hidden > 0, "rmsnorm_wide: bad sizes rows=%d hidden=%d", nrows, hidden);
-  PA_REQUIRE((x != nullptr) != (parts != nullptr), "rmsnorm_wide: give x or partial sums (one of them)");
+  PA_REQUIRE(!(x && parts) && (x || parts || (residual && rows)),
+             "rmsnorm_wide: give x or partial sums (one of them), or the residual and the rows to norm alone");
   PA_REQUIRE(!parts || slices >= 1, "rmsnorm_wide: %d slices", slices);
   hipStream_t st = (hipStream_t)stream;
   if (dtype == kF32)
@@ -190,4 +307,36 @@ extern "C" int pa_relu_squared(void* stream, int dtype, const void* x, void* out
   else
     return pa::fail("relu_squared: unknown element type code %d", dtype);
   return check_launch("relu_squared");
+}
+
+extern "C" int pa_rmsnorm_branch(void* stream, int dtype, const void* x, const float* parts, int slices, long slice_stride,
+                                 float* residual, const float* w, void* copy, int nrows, int hidden, float eps) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && hidden > 0 && residual && w, "rmsnorm_branch: bad sizes rows=%d hidden=%d", nrows, hidden);
+  PA_REQUIRE((x != nullptr) != (parts != nullptr), "rmsnorm_branch: give x or partial sums (one of them)");
+  PA_REQUIRE(!parts || slices >= 1, "rmsnorm_branch: %d slices", slices);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == kF32)
+    launch_branch<float>(st, (const float*)x, parts, slices, (size_t)slice_stride, residual, w, (float*)copy, nrows, hidden, eps);
+  else if (dtype == kBF16)
+    launch_branch<bf16>(st, (const bf16*)x, parts, slices, (size_t)slice_stride, residual, w, (bf16*)copy, nrows, hidden, eps);
+  else
+    return pa::fail("rmsnorm_branch: unknown element type code %d", dtype);
+  return check_launch("rmsnorm_branch");
+}
+
+extern "C" int pa_gated_rmsnorm(void* stream, int dtype, const float* o, const void* gate, long gate_stride, const float* w,
+                                void* out, int nrows, int width, float eps) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && width > 0 && gate_stride >= width, "gated_rmsnorm: bad sizes rows=%d width=%d gate stride=%ld", nrows,
+             width, gate_stride);
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (dtype == kF32)
+    rc = launch_gated<float>(st, o, (const float*)gate, (size_t)gate_stride, w, (float*)out, nrows, width, eps);
+  else if (dtype == kBF16)
+    rc = launch_gated<bf16>(st, o, (const bf16*)gate, (size_t)gate_stride, w, (bf16*)out, nrows, width, eps);
+  else
+    return pa::fail("gated_rmsnorm: unknown element type code %d", dtype);
+  return rc ? rc : check_launch("gated_rmsnorm");
 }

@@ -167,6 +167,10 @@ class CausalLM:
                                                             write_cache=r.reads_cache_of is None)
         if step.want_rows.shape[0] == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=hidden.device)
+        if self.blocks[self.spec.order[-1].layer].HANDS_ON_STREAM:
+            # the last block handed on the stream itself: nothing waits to be added, the norm is of its rows alone
+            normed = self.final_norm.forward_rows(None, residual, step.want_rows, out_dtype=hidden.dtype)
+            return self.head.forward(normed)
         if not self.final_norm.TAKES_SLICE_SUMS:
             from ..ops import kernels as K
             hidden = K.as_tensor(hidden)

@@ -210,21 +210,26 @@ def _check_caches(k_cache, v_cache, num_kv_heads, head_dim, dtype, what) -> None
 def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
                    cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                    slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                   num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int, eps: float) -> torch.Tensor:
+                   num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int, eps: float,
+                   inv_freq: Optional[torch.Tensor] = None, values_from_keys: bool = False) -> torch.Tensor:
     """Per-head RMSNorm of Q and K, rotation by position, K and V into the paged cache.
 
     qkv [T, (nh + 2 nkv) * hd]; returns q [T, nh, hd].  With ``slots`` None
     nothing is written to the cache (then ``num_kv_heads`` may be 0 for a
     Q-only input).  K cache [pages, nkv, page_size, hd], V cache [pages, nkv, hd, page_size].
+    ``inv_freq`` (float32 [rotary_dim / 2]) in place of the tables: the kernel takes the angle
+    position * inv_freq[j] and its cosine and sine itself.  ``values_from_keys``: qkv is [T, (nh + nkv) * hd]
+    and a head's cached value is its key as projected, before norm and rotation.
     """
-    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache)
+    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, inv_freq)
     _i32(positions, "positions")
     _f32(q_weight, "q_norm weight")
     _f32(k_weight, "k_norm weight")
     _f32(cos, "cos table")
     _f32(sin, "sin table")
+    _f32(inv_freq, "rotary frequencies")
     t = qkv.shape[0]
-    width = (num_heads + 2 * num_kv_heads) * head_dim
+    width = (num_heads + (1 if values_from_keys else 2) * num_kv_heads) * head_dim
     if qkv.dim() != 2 or qkv.shape[1] != width:
         raise NativeError(f"qknorm_rope_kv: qkv {tuple(qkv.shape)} is not [T, {width}]")
     if positions.shape != (t,):
@@ -232,7 +237,13 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
     for w, nm in ((q_weight, "q_norm"), (k_weight, "k_norm")):
         if w is not None and w.shape != (head_dim,):
             raise NativeError(f"qknorm_rope_kv: {nm} weight {tuple(w.shape)} is not [{head_dim}]")
-    if rotary_dim:
+    by_freq = inv_freq is not None or values_from_keys
+    if rotary_dim and inv_freq is not None:
+        if cos is not None or sin is not None or tuple(inv_freq.shape) != (rotary_dim // 2,):
+            raise NativeError(f"qknorm_rope_kv: frequencies must be [{rotary_dim // 2}] and come without tables")
+    elif rotary_dim:
+        if values_from_keys:
+            raise NativeError("qknorm_rope_kv: values that are the keys are rotated from the frequencies, not from tables")
         if cos is None or sin is None or cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != rotary_dim // 2:
             raise NativeError(f"qknorm_rope_kv: cos/sin tables must be [positions, {rotary_dim // 2}]")
     page_size = 1
@@ -243,6 +254,12 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
         _check_caches(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, "qknorm_rope_kv")
         page_size = k_cache.shape[2]
     q_out = torch.empty((t, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    if by_freq:
+        check(kernels().pa_qknorm_rope_kv_freq(_stream(), _code(qkv), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(inv_freq),
+                                               _ptr(positions), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), t,
+                                               num_heads, num_kv_heads, head_dim, rotary_dim, page_size, float(eps),
+                                               1 if values_from_keys else 0))
+        return q_out
     check(kernels().pa_qknorm_rope_kv(_stream(), _code(qkv), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos),
                                       _ptr(sin), _ptr(positions), _ptr(slots), _ptr(q_out), _ptr(k_cache),
                                       _ptr(v_cache), t, num_heads, num_kv_heads, head_dim, rotary_dim, page_size,
@@ -786,8 +803,9 @@ def linear_silu_mul(x: torch.Tensor, w) -> torch.Tensor:
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       seq_of_token: torch.Tensor, positions: torch.Tensor, window: int, scale: float,
-                      softcap: float = 0.0) -> torch.Tensor:
-    """Paged causal attention, any mix of portions and decode tokens.  ``softcap`` > 0 (here and in the other
+                      softcap: float = 0.0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Paged causal attention, any mix of portions and decode tokens.  ``sink`` (float32 [heads], here and in
+    ``attention``): a head's softmax divides by sum_j exp(score_j) + exp(sink_h), a term that brings no value.  ``softcap`` > 0 (here and in the other
     attention entry points) bends every scaled score to ``softcap * tanh(score / softcap)`` before the softmax;
     0, the default, leaves the scores alone (the same bits as without the parameter).
 
@@ -806,6 +824,16 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if seq_of_token.shape != (t,) or positions.shape != (t,) or block_table.dim() != 2:
         raise NativeError("attention: index arrays do not match the number of tokens")
     out = torch.empty_like(q)
+    if sink is not None:
+        _dev(sink)
+        _f32(sink, "sinks")
+        if tuple(sink.shape) != (nh,):
+            raise NativeError(f"attention: sinks {tuple(sink.shape)} for {nh} heads")
+        check(kernels().pa_attn_generic_sink(_stream(), _code(q), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+                                             block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out), t, nh,
+                                             k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale),
+                                             float(softcap), _ptr(sink)))
+        return out
     check(kernels().pa_attn_generic(_stream(), _code(q), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
                                     block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out), t, nh,
                                     k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale), float(softcap)))
@@ -946,7 +974,7 @@ def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_l
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, step, window: int,
-              scale: float, softcap: float = 0.0) -> torch.Tensor:
+              scale: float, softcap: float = 0.0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of one step over one cache group; picks the kernel for the sizes at hand.
 
     ``group`` is the step's ``GroupStep`` of the cache group, ``step`` the ``StepBatch``.
@@ -954,7 +982,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
     tokens go to the split decode kernel, portions to the prefill kernel.
     Everything else (float32, other sizes) goes to the generic kernel.
     """
-    if q.dtype == torch.bfloat16 and step.decode_seqs is not None \
+    if q.dtype == torch.bfloat16 and step.decode_seqs is not None and sink is None \
             and mfma_attention_supported(q.shape[2], k_cache.shape[2]):
         out = torch.empty_like(q)
         if step.n_decode:
@@ -966,7 +994,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
                               out, step.max_prefill_q, window, scale, min_prefix=step.min_prefill_prefix, softcap=softcap)
         return out
     return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale,
-                             softcap)
+                             softcap, sink)
 
 
 def logprobs(logits: torch.Tensor, ids: torch.Tensor, k: int = 0):
@@ -1041,7 +1069,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
 # ---------------------------------------------------------------------------
 # A residual stream kept in 32-bit
 def rmsnorm_wide(x, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None,
-                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 rows: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``rmsnorm`` for a float32 residual [T, H] beside x [T, H] of the engine's type (or a ``SliceSums``): the sum
     is taken and kept in 32-bit (the residual receives it unrounded, unless ``rows``), the output is of x's type."""
     parts = x.parts if isinstance(x, SliceSums) else None
@@ -1049,6 +1077,15 @@ def rmsnorm_wide(x, weight: torch.Tensor, eps: float, residual: Optional[torch.T
     _dev(xt, parts, weight, residual, rows)
     _f32(weight, "norm weight")
     _f32(residual, "residual")
+    if x is None:
+        # nothing waits to be added: the norm of the stream's wanted rows alone, in ``out_dtype``
+        if residual is None or rows is None or out_dtype is None:
+            raise NativeError("rmsnorm_wide: without x it norms rows of the residual and needs residual, rows and out_dtype")
+        _i32(rows, "rows")
+        out = torch.empty((rows.shape[0], residual.shape[1]), dtype=out_dtype, device=weight.device)
+        check(kernels().pa_rmsnorm_wide(_stream(), _CODES[out_dtype], None, None, 0, 0, _ptr(residual), _ptr(weight), _ptr(out),
+                                        _ptr(rows), rows.shape[0], residual.shape[1], float(eps)))
+        return out
     m, h = x.shape
     if weight.shape != (h,) or (residual is not None and tuple(residual.shape) != (m, h)):
         raise NativeError(f"rmsnorm_wide: x {tuple(x.shape)} / weight {tuple(weight.shape)} / residual "
@@ -1061,6 +1098,73 @@ def rmsnorm_wide(x, weight: torch.Tensor, eps: float, residual: Optional[torch.T
     check(kernels().pa_rmsnorm_wide(_stream(), _CODES[x.dtype], _ptr(xt), _ptr(parts),
                                     0 if parts is None else parts.shape[0], m * h, _ptr(residual), _ptr(weight), _ptr(out),
                                     _ptr(rows), n, h, float(eps)))
+    return out
+
+
+def rmsnorm_branch(y, weight: torch.Tensor, eps: float, residual: torch.Tensor,
+                   copy_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """residual += y / sqrt(mean(y^2) + eps) * weight, in 32-bit and in place: a branch's output normed and added to
+    the stream.  y [T, H] of the engine's type or a ``SliceSums``; residual float32 [T, H].  Returns the new residual
+    rounded to ``copy_dtype`` (what the next branch multiplies with), or None when that is float32 itself."""
+    parts = y.parts if isinstance(y, SliceSums) else None
+    yt = None if parts is not None else y
+    _dev(yt, parts, weight, residual)
+    _f32(weight, "norm weight")
+    _f32(residual, "residual")
+    m, h = y.shape
+    if weight.shape != (h,) or tuple(residual.shape) != (m, h):
+        raise NativeError(f"rmsnorm_branch: y {tuple(y.shape)} / weight {tuple(weight.shape)} / residual {tuple(residual.shape)}")
+    copy = None
+    if copy_dtype is not None and copy_dtype != torch.float32:
+        if copy_dtype != y.dtype:
+            raise NativeError(f"rmsnorm_branch: a copy of {copy_dtype} beside a branch of {y.dtype}")
+        copy = torch.empty((m, h), dtype=copy_dtype, device=residual.device)
+    check(kernels().pa_rmsnorm_branch(_stream(), _CODES[y.dtype], _ptr(yt), _ptr(parts), 0 if parts is None else parts.shape[0],
+                                      m * h, _ptr(residual), _ptr(weight), _ptr(copy), m, h, float(eps)))
+    return copy
+
+
+def gated_rmsnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """out = o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate) over rows; o float32 [T, N]; gate [T, N] of the engine's
+    type, a view whose rows may lie inside a wider tensor (columns contiguous); the output is of the gate's type."""
+    _dev(o, weight)
+    _f32(o, "gated_rmsnorm input")
+    _f32(weight, "norm weight")
+    if not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1 or o.dim() != 2 or gate.shape != o.shape \
+            or weight.shape != (o.shape[1],):
+        raise NativeError(f"gated_rmsnorm: o {tuple(o.shape)} / gate {tuple(gate.shape)} strides {gate.stride()} / weight "
+                          f"{tuple(weight.shape)}")
+    out = torch.empty(o.shape, dtype=gate.dtype, device=o.device)
+    check(kernels().pa_gated_rmsnorm(_stream(), _code(gate), _ptr(o), gate.data_ptr(), gate.stride(0), _ptr(weight), _ptr(out),
+                                     o.shape[0], o.shape[1], float(eps)))
+    return out
+
+
+LIGHTNING_ACTIVATIONS = {None: 0, "none": 0, "silu": 1}
+
+
+def lightning_attention(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, state: torch.Tensor,
+                        step, heads: int, dim: int, vdim: int, activation: Optional[str] = "silu") -> torch.Tensor:
+    """Linear attention with a decaying state: per head S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t.
+
+    qkv [T, width]: a token's queries [heads, dim], keys [heads, dim] and values [heads, vdim] start at columns
+    ``q_off``, ``k_off``, ``v_off`` and pass through ``activation``; decay float32 [heads]; state float32
+    [slots, heads, dim, vdim], read and left by the step's sequences through ``step.state_slots``.  Returns
+    float32 [T, heads, vdim]."""
+    _dev(qkv, decay, state)
+    _f32(decay, "decays")
+    _f32(state, "state")
+    t = qkv.shape[0]
+    if qkv.dim() != 2 or tuple(decay.shape) != (heads,) or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim) \
+            or max(q_off, k_off) + heads * dim > qkv.shape[1] or v_off + heads * vdim > qkv.shape[1]:
+        raise NativeError(f"lightning_attention: qkv {tuple(qkv.shape)} / decay {tuple(decay.shape)} / state {tuple(state.shape)} "
+                          f"for {heads} heads of {dim} and {vdim}")
+    if activation not in LIGHTNING_ACTIVATIONS:
+        raise NativeError(f"lightning_attention: activation {activation!r} is not one of {sorted(map(str, LIGHTNING_ACTIVATIONS))}")
+    out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qkv.device)
+    check(kernels().pa_lightning_attn(_stream(), _code(qkv), _ptr(qkv), qkv.shape[1], int(q_off), int(k_off), int(v_off),
+                                      _ptr(decay), _ptr(state), _ptr(step.state_slots), _ptr(step.cu_q), _ptr(out),
+                                      step.num_seqs, t, heads, dim, vdim, LIGHTNING_ACTIVATIONS[activation]))
     return out
 
 
@@ -1218,6 +1322,26 @@ def moe_choices_by_table(token_ids: torch.Tensor, table: torch.Tensor, experts: 
     return choice
 
 
+def moe_route(logits: torch.Tensor, experts: int, top: int, scale: float, correction: Optional[torch.Tensor] = None,
+              gate_col: int = -1):
+    """A router's choices: logits float32 [T, >= experts]; s = softmax over the first ``experts`` columns; the ``top``
+    experts with the largest s + correction are chosen and weighted s / (sum of the chosen s + 1e-20) * scale.
+    Returns (choice int32 [T * top], weights float32 [T * top], gate float32 [T] or None): the gate is the sigmoid of
+    column ``gate_col`` of the same rows, for a shared expert."""
+    _dev(logits, correction)
+    _f32(logits, "router logits")
+    _f32(correction, "router correction")
+    if logits.dim() != 2 or logits.shape[1] < experts or (correction is not None and tuple(correction.shape) != (experts,)):
+        raise NativeError(f"moe_route: logits {tuple(logits.shape)} for {experts} experts")
+    t = logits.shape[0]
+    choice = torch.empty(t * top, dtype=torch.int32, device=logits.device)
+    weights = torch.empty(t * top, dtype=torch.float32, device=logits.device)
+    gate = torch.empty(t, dtype=torch.float32, device=logits.device) if gate_col >= 0 else None
+    check(kernels().pa_moe_route(_stream(), _ptr(logits), logits.shape[1], _ptr(correction), _ptr(choice), _ptr(weights),
+                                 _ptr(gate), t, int(experts), int(top), float(scale), int(gate_col)))
+    return choice, weights, gate
+
+
 def moe_order(choice: torch.Tensor, experts: int, top: int) -> ExpertOrder:
     _dev(choice)
     _i32(choice, "choices")
@@ -1251,19 +1375,20 @@ def moe_linear(x: torch.Tensor, w: GroupedWeight, eo: ExpertOrder, from_tokens: 
 
 
 def moe_combine(y: torch.Tensor, eo: ExpertOrder, weight: float, base: Optional[torch.Tensor], out_dtype: torch.dtype,
-                weights: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = base[t] + sum_j w * y[place[t * top + j]] in ascending j; y float32 [entries, H]; ``weights`` float32
-    [entries] per entry, else ``weight`` for all."""
-    _dev(y, base, weights)
+                weights: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = b[t] * base[t] + sum_j w * y[place[t * top + j]] in ascending j; y float32 [entries, H]; ``weights``
+    float32 [entries] per entry, else ``weight`` for all; ``base_scale`` float32 [T] gives b, else 1."""
+    _dev(y, base, weights, base_scale)
     _f32(y, "expert outputs")
     _f32(weights, "entry weights")
+    _f32(base_scale, "base scale")
     t = eo.entries // eo.top
     h = y.shape[1]
     if y.shape[0] != eo.entries or (base is not None and (tuple(base.shape) != (t, h) or base.dtype != out_dtype)):
         raise NativeError(f"moe_combine: y {tuple(y.shape)} / base {None if base is None else tuple(base.shape)}")
     out = torch.empty((t, h), dtype=out_dtype, device=y.device)
     check(kernels().pa_moe_combine(_stream(), _CODES[out_dtype], _ptr(y), _ptr(eo.place), _ptr(weights), float(weight), _ptr(base),
-                                   _ptr(out), t, eo.top, h))
+                                   _ptr(base_scale), _ptr(out), t, eo.top, h))
     return out
 
 

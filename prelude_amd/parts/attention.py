@@ -1,5 +1,5 @@
 """Grouped-query attention over a paged cache, with optional per-head QK norm,
-rotary encoding, biases and a window.
+rotary encoding, biases and a window; optionally with the keys as projected for values and a sink in the softmax.
 
 One merged projection [(nh + 2 nkv) hd, H] (crates/prelude-core/src/models/qwen3.rs:89-106,
 crates/prelude-core/src/models/commons/attn_utils.rs:91-133; unlike the
@@ -27,7 +27,8 @@ class GQAAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, norm_eps: float = 1e-6,
                  qk_norm: bool = True, bias: bool = False, window: int = 0, position: Optional[str] = None,
-                 rotary_dim: Optional[int] = None, scale: Optional[float] = None, score_cap: float = 0.0):
+                 rotary_dim: Optional[int] = None, scale: Optional[float] = None, score_cap: float = 0.0,
+                 values_from_keys: bool = False, sink: Optional[str] = None):
         if num_heads % num_kv_heads:
             raise PartError(f"gqa_attention: {num_heads} heads are not a multiple of {num_kv_heads} KV heads")
         # what the kernels take: the matrix-core attention has head sizes of its own (others go to the generic
@@ -44,8 +45,18 @@ class GQAAttention(Mixer):
         self.score_cap = float(score_cap or 0.0)
         if self.score_cap < 0:
             raise PartError(f"gqa_attention: a score cap of {score_cap} is negative")
+        # the values are the keys as projected (before norm and rotation): there is no value projection, and the
+        # merged product has nh + nkv heads
+        self.values_from_keys = bool(values_from_keys)
+        # one more term of the softmax's denominator that brings no value: "zero" exp(0) = 1 for every head,
+        # "learned" exp(s_h) with a tensor ``sinks`` [heads] (in the units of the scaled scores); None: none
+        if sink not in (None, "zero", "learned"):
+            raise PartError(f"gqa_attention: sink {sink!r} is not one of None, 'zero', 'learned'")
+        self.sink = sink
+        if self.values_from_keys and self.bias:
+            raise PartError("gqa_attention: values that are the keys come without biases")
         self.rope = None
-        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = None
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = self.sinks = None
 
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
@@ -55,6 +66,9 @@ class GQAAttention(Mixer):
             if self.position not in shared:
                 raise PartError(f"gqa_attention: the model has no position encoding named {self.position!r}")
             self.rope = shared[self.position]
+            if self.values_from_keys and not hasattr(self.rope, "inv_freq"):
+                raise PartError("gqa_attention: values that are the keys take their rotation from frequencies "
+                                "(a position encoding that offers `inv_freq`), not from tables")
             if getattr(self.rope, "rotary_dim", None) != self.rotary_dim:
                 raise PartError(f"gqa_attention: position encoding {self.position!r} has width "
                                 f"{getattr(self.rope, 'rotary_dim', None)}, the mixer rotates {self.rotary_dim}")
@@ -63,6 +77,10 @@ class GQAAttention(Mixer):
         h, nh, nkv, hd = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
         t = {"q_proj.weight": TensorReq((nh * hd, h), MATRIX), "k_proj.weight": TensorReq((nkv * hd, h), MATRIX),
              "v_proj.weight": TensorReq((nkv * hd, h), MATRIX), "o_proj.weight": TensorReq((h, nh * hd), MATRIX)}
+        if self.values_from_keys:
+            del t["v_proj.weight"]
+        if self.sink == "learned":
+            t["sinks"] = TensorReq((nh,), VECTOR)
         if self.bias:
             t.update({"q_proj.bias": TensorReq((nh * hd,), VECTOR), "k_proj.bias": TensorReq((nkv * hd,), VECTOR),
                       "v_proj.bias": TensorReq((nkv * hd,), VECTOR), "o_proj.bias": TensorReq((h,), VECTOR)})
@@ -71,8 +89,14 @@ class GQAAttention(Mixer):
         return t
 
     def load(self, tensors, dtype, device):
-        self.w_qkv = K.prepare_weight(torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
-                                                 tensors["v_proj.weight"]], dim=0).contiguous())
+        merged = [tensors["q_proj.weight"], tensors["k_proj.weight"]]
+        if not self.values_from_keys:
+            merged.append(tensors["v_proj.weight"])
+        self.w_qkv = K.prepare_weight(torch.cat(merged, dim=0).contiguous())
+        if self.sink == "learned":
+            self.sinks = tensors["sinks"]
+        elif self.sink == "zero":
+            self.sinks = torch.zeros(self.num_heads, dtype=torch.float32, device=device)
         self.w_o = K.prepare_weight(tensors["o_proj.weight"])
         if self.bias:
             self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]).contiguous()
@@ -86,6 +110,7 @@ class GQAAttention(Mixer):
         """Few sequences, each feeding one token: a kernel less per layer counts for more than the norm and the
         rotation that every workgroup of the attention kernel then does for itself."""
         return (x.dtype == torch.bfloat16 and self.rope is not None and step.decode_seqs is not None
+                and getattr(self.rope, "cos", None) is not None and not self.values_from_keys and self.sinks is None
                 and step.n_prefill == 0 and step.n_decode == step.num_seqs <= self.FUSED_DECODE_MAX_SEQS
                 and K.attention_decode_fused_supported(self.num_heads, self.num_kv_heads, self.head_dim,
                                                        self.rotary_dim, cache.k.shape[2]))
@@ -93,8 +118,11 @@ class GQAAttention(Mixer):
     def forward(self, x, step, cache, write_cache=True):
         nh, nkv, hd = self.num_heads, self.num_kv_heads, self.head_dim
         g = step.kv[cache.group]
-        cos = self.rope.cos if self.rope is not None else None
-        sin = self.rope.sin if self.rope is not None else None
+        # tables by position, or the frequencies alone (the kernel then takes angle, cosine and sine itself)
+        cos = getattr(self.rope, "cos", None) if self.rope is not None else None
+        sin = getattr(self.rope, "sin", None) if self.rope is not None else None
+        freq = getattr(self.rope, "inv_freq", None) if self.rope is not None and cos is None else None
+        how = dict(inv_freq=freq, values_from_keys=self.values_from_keys) if (freq is not None or self.values_from_keys) else {}
         if write_cache and self._fused_decode(x, step, cache):
             # a step of single tokens: the norm, the rotation and the cache write happen inside the attention kernel
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
@@ -106,11 +134,11 @@ class GQAAttention(Mixer):
         if write_cache:
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
             q = K.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, cos, sin, step.positions, g.slots, cache.k, cache.v,
-                                 nh, nkv, hd, self.rotary_dim, self.norm_eps)
+                                 nh, nkv, hd, self.rotary_dim, self.norm_eps, **how)
         else:  # reads keys and values another layer wrote: only the queries are projected
             bq = self.b_qkv[: nh * hd] if self.b_qkv is not None else None
             qx = K.linear(x, self.w_qkv.first_rows(nh * hd), bq)
             q = K.qknorm_rope_kv(qx, self.q_norm, None, cos, sin, step.positions, None, None, None, nh, 0, hd,
-                                 self.rotary_dim, self.norm_eps)
-        o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale, self.score_cap)
+                                 self.rotary_dim, self.norm_eps, **({"inv_freq": freq} if freq is not None else {}))
+        o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale, self.score_cap, sink=self.sinks)
         return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o, slices_ok=True)

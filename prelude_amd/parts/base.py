@@ -8,7 +8,7 @@ tensors it needs (by local name and shape), receives them, and runs.
 Categories and the interface each must have:
 
 ``norm``      ``forward(x)``, ``forward_residual(x, residual) -> (residual, normed)``,
-              ``forward_rows(x, residual, rows)``; ``as_rms() -> (gain, eps) | None`` (given by the base class:
+              ``forward_rows(x, residual, rows)``; for blocks that norm a branch's output, ``forward_branch``; ``as_rms() -> (gain, eps) | None`` (given by the base class:
               None) tells a kernel behind it that it may do the plain RMS formula itself
 ``mixer``/``ffn`` may return their last product as ``ops.kernels.SliceSums`` (``linear(..., slices_ok=True)``):
               only a norm reads it, and one that says ``TAKES_SLICE_SUMS`` adds the slices itself
@@ -276,6 +276,13 @@ class Norm(Part):
     def forward_rows(self, x: torch.Tensor, residual: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
+    def forward_branch(self, y, residual: torch.Tensor, copy_dtype=None):
+        """For a block whose norms sit on the branches' outputs: residual += norm(y) in place (a 32-bit stream);
+        returns a copy of the new residual in ``copy_dtype``, or None when that is the residual's own type.  A norm
+        that is to be the final norm behind such a block also takes ``forward_rows(None, residual, rows,
+        out_dtype=)``: the norm of the stream's rows alone."""
+        raise NotImplementedError
+
 
 class PositionEncoding(Part):
     def prepare(self, device: torch.device) -> None:
@@ -286,6 +293,10 @@ class Block(Part):
     """An arrangement of parts.  ``SLOTS`` names the sub-parts it is built from: slot -> category."""
     SLOTS: Dict[str, str] = {}
     LAUNCHES = 0   # of the arrangement itself; its sub-parts count their own
+    # What the ``hidden`` a block hands on means.  False: a branch's output that the next norm still has to add to
+    # the residual.  True: the stream itself (the residual, or its copy in the engine's type), with nothing left to
+    # add: the final norm then norms the residual's wanted rows alone.
+    HANDS_ON_STREAM = False
 
     def forward(self, hidden, residual, step, cache, write_cache: bool = True):
         raise NotImplementedError

@@ -4,8 +4,14 @@
 residual carried beside the hidden state and each add deferred into the next
 norm (crates/prelude-core/src/models/qwen3.rs:486-502,
 crates/prelude-core/src/models/commons/linear.rs:471-488).
+
+``branch_norm``: the norm sits on each branch's output, x <- x + norm(mixer(x)) and x <- x + norm(ffn(x)); the
+branches read the stream itself.  The stream is 32-bit; beside it travels its copy in the engine's type, which is
+what the branches multiply with.
 """
 from __future__ import annotations
+
+import torch
 
 from ..ops import kernels as K
 from .base import Block, register_part
@@ -49,3 +55,54 @@ class PreNormMixerBlock(Block):
             hidden = K.as_tensor(hidden)
         residual, h = self.input_norm.forward_residual(hidden, residual)
         return self.mixer.forward(h, step, cache, write_cache), residual
+
+
+@register_part("block", "branch_norm")
+class BranchNormBlock(Block):
+    """x <- x + mixer_norm(mixer(x)); x <- x + ffn_norm(ffn(x)).  Both branches read x itself, the norms sit on their
+    outputs, and the sums are taken and kept in 32-bit.  ``hidden`` carried between such blocks is x in the engine's
+    type (the residual itself in a 32-bit engine), written by the kernel that norms and adds."""
+    GRAPH_SAFE_PORTIONS = True
+    HANDS_ON_STREAM = True
+
+    SLOTS = {"mixer": "mixer", "mixer_norm": "norm", "ffn": "ffn", "ffn_norm": "norm"}
+
+    def __init__(self, mixer, mixer_norm, ffn, ffn_norm):
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = mixer, mixer_norm, ffn, ffn_norm
+
+    @staticmethod
+    def _enter(hidden, residual):
+        if residual is None:   # the first block: the stream starts as a 32-bit copy of the embedding
+            hidden = K.as_tensor(hidden)
+            residual = hidden if hidden.dtype == torch.float32 else K.to_f32(hidden)
+        return hidden, residual
+
+    @staticmethod
+    def _add(norm, y, hidden, residual):
+        if not norm.TAKES_SLICE_SUMS:
+            y = K.as_tensor(y)
+        copy = norm.forward_branch(y, residual, hidden.dtype)
+        return residual if copy is None else copy
+
+    def forward(self, hidden, residual, step, cache, write_cache=True):
+        hidden, residual = self._enter(hidden, residual)
+        hidden = self._add(self.mixer_norm, self.mixer.forward(hidden, step, cache, write_cache), hidden, residual)
+        y = self.ffn.forward(hidden, step=step) if getattr(self.ffn, "NEEDS_STEP", False) else self.ffn.forward(hidden)
+        return self._add(self.ffn_norm, y, hidden, residual), residual
+
+
+@register_part("block", "branch_norm_mixer_only")
+class BranchNormMixerBlock(Block):
+    """A ``branch_norm`` layer without a feed-forward: x <- x + mixer_norm(mixer(x))."""
+    GRAPH_SAFE_PORTIONS = True
+    HANDS_ON_STREAM = True
+
+    SLOTS = {"mixer": "mixer", "mixer_norm": "norm"}
+
+    def __init__(self, mixer, mixer_norm):
+        self.mixer, self.mixer_norm = mixer, mixer_norm
+
+    def forward(self, hidden, residual, step, cache, write_cache=True):
+        hidden, residual = BranchNormBlock._enter(hidden, residual)
+        y = self.mixer.forward(hidden, step, cache, write_cache)
+        return BranchNormBlock._add(self.mixer_norm, y, hidden, residual), residual

@@ -1,4 +1,5 @@
-"""A feed-forward of many small experts, of which every token uses a few.
+"""Feed-forwards of many small experts, of which every token uses a few: chosen from a table by token id
+(``table_experts``) or by a router's scores (``routed_experts``, at the end of this file).
 
 An expert is down(act(up(x))) without biases, act the square of relu.  Which experts a token uses is read from
 a table by its token id (``table_experts``: a row of ``top`` distinct experts per id, each weighted 1 / top;
@@ -15,7 +16,7 @@ from typing import Optional
 import torch
 
 from ..ops import kernels as K
-from .base import MATRIX, TABLE, FeedForward, PartError, TensorReq, register_part
+from .base import MATRIX, TABLE, VECTOR, FeedForward, PartError, TensorReq, register_part
 
 
 @register_part("ffn", "table_experts")
@@ -65,3 +66,80 @@ class TableExperts(FeedForward):
         if self.shared_size:
             base = K.as_tensor(K.linear(K.relu_squared(K.linear(x, self.shared_up)), self.shared_down))
         return K.moe_combine(y, eo, 1.0 / self.top, base, x.dtype)
+
+
+@register_part("ffn", "routed_experts")
+class RoutedExperts(FeedForward):
+    """Experts chosen by a router.  Scores s = softmax(W_router x) over all experts, in 32-bit; a token's ``top``
+    experts are those with the largest s + correction (a stored vector that bears on the choice alone); their
+    weights are their s over the chosen ones' sum (+ 1e-20), times ``route_scale``.  An expert is a gated pair with
+    both halves clamped, down(g * sigmoid(alpha g) * (u + 1)) with g = min(gate(x), limit) and u = clamp(up(x),
+    -limit, limit), without biases.  An optional shared expert of the same form (its own size and limit) runs for
+    every token and is added times sigmoid(w_sg . x), one number a token.
+
+    The router and the shared expert's gate are one product ([experts + 1, hidden]) whose 32-bit sums one kernel turns
+    into choices, weights and gates; from there on the path is that of ``table_experts``: entries in the order of
+    their experts, two grouped products, the outputs added per token in the order of its choices.  Nothing is decided
+    on the host."""
+    LAUNCHES = 12
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, limit: float, route_scale: float = 1.0,
+                 alpha: float = 1.702, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0):
+        if not 1 <= int(top) <= int(num_experts):
+            raise PartError(f"routed_experts: {top} of {num_experts} experts a token")
+        if not limit > 0 or (shared_size and not shared_limit > 0):
+            raise PartError(f"routed_experts: the clamps {limit} and {shared_limit} must be positive")
+        self.hidden_size, self.num_experts, self.top = int(hidden_size), int(num_experts), int(top)
+        self.expert_size, self.limit, self.alpha = int(expert_size), float(limit), float(alpha)
+        self.route_scale, self.has_correction = float(route_scale), bool(correction)
+        self.shared_size, self.shared_limit = int(shared_size or 0), float(shared_limit or 0.0)
+        self.router = self.correction = self.gate_up_t = self.down_t = None
+        self.shared_gate_up = self.shared_down = None
+
+    def tensors(self):
+        h, f, n = self.hidden_size, self.expert_size, self.num_experts
+        t = {"router": TensorReq((n, h), MATRIX)}
+        if self.has_correction:
+            t["correction"] = TensorReq((n,), VECTOR)
+        for e in range(n):
+            t[f"e{e}.gate"] = TensorReq((f, h), MATRIX)
+            t[f"e{e}.up"] = TensorReq((f, h), MATRIX)
+            t[f"e{e}.down"] = TensorReq((h, f), MATRIX)
+        if self.shared_size:
+            s = self.shared_size
+            t.update({"shared.gate": TensorReq((s, h), MATRIX), "shared.up": TensorReq((s, h), MATRIX),
+                      "shared.down": TensorReq((h, s), MATRIX), "shared.sg": TensorReq((1, h), MATRIX)})
+        return t
+
+    @staticmethod
+    def _pairs(gate, up):
+        """Rows alternating gate_j, up_j: one product yields each pair side by side."""
+        return torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
+
+    def load(self, tensors, dtype, device):
+        n = self.num_experts
+        rows = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_size else [])
+        self.router = torch.cat(rows, dim=0).contiguous()
+        self.correction = tensors["correction"] if self.has_correction else None
+        self.gate_up_t = K.GroupedWeight(torch.stack([self._pairs(tensors[f"e{e}.gate"], tensors[f"e{e}.up"]) for e in range(n)]))
+        self.down_t = K.GroupedWeight(torch.stack([tensors[f"e{e}.down"] for e in range(n)]))
+        if self.shared_size:
+            self.shared_gate_up = K.prepare_weight(self._pairs(tensors["shared.gate"], tensors["shared.up"]))
+            self.shared_down = K.prepare_weight(tensors["shared.down"])
+
+    def forward(self, x, step=None):
+        n = self.num_experts
+        # the router's sums are 32-bit in a fixed order whatever the number of rows (the operands are of the engine's
+        # type): a product of few columns, for which the plain kernel is the right one
+        logits = K.gemm_plain(x, self.router, None, torch.float32)
+        choice, weights, gate = K.moe_route(logits, n, self.top, self.route_scale, self.correction,
+                                            gate_col=n if self.shared_size else -1)
+        eo = K.moe_order(choice, n, self.top)
+        mid = K.clamped_gate(K.moe_linear(x, self.gate_up_t, eo, from_tokens=True), self.limit, self.alpha)
+        y = K.moe_linear(mid, self.down_t, eo, from_tokens=False, out_dtype=torch.float32)
+        base: Optional[torch.Tensor] = None
+        if self.shared_size:
+            base = K.as_tensor(K.linear(K.linear_clamped_gate(x, self.shared_gate_up, self.shared_limit, self.alpha),
+                                        self.shared_down))
+        return K.moe_combine(y, eo, 1.0, base, x.dtype, weights=weights, base_scale=gate)

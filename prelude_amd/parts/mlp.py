@@ -81,3 +81,24 @@ class ClampedGatedMLP(FeedForward):
 
     def forward(self, x):
         return K.linear(K.linear_clamped_gate(x, self.gate_up, self.limit, self.alpha), self.down, slices_ok=True)
+
+
+@register_part("ffn", "squared_relu_mlp")
+class SquaredReluMLP(FeedForward):
+    """down(relu(up(x))^2): two products and the square of relu between them, no gate and no biases."""
+    LAUNCHES = 3
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.up = self.down = None
+
+    def tensors(self):
+        h, i = self.hidden_size, self.intermediate_size
+        return {"up": TensorReq((i, h), MATRIX), "down": TensorReq((h, i), MATRIX)}
+
+    def load(self, tensors, dtype, device):
+        self.up, self.down = K.prepare_weight(tensors["up"]), K.prepare_weight(tensors["down"])
+
+    def forward(self, x):
+        return K.linear(K.relu_squared(K.linear(x, self.up)), self.down, slices_ok=True)

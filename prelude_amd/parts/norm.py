@@ -1,4 +1,4 @@
-"""RMSNorm, alone or fused with the residual add.
+"""RMSNorm, alone, fused with the residual add in front of it, or on a branch's output with the add behind it.
 
 y = x * rsqrt(mean(x^2) + eps) * w in 32-bit
 (crates/prelude-core/src/models/commons/linear.rs:435-501); with a residual:
@@ -61,7 +61,19 @@ class RMSNorm(Norm):
         out = K.rmsnorm(x, self.weight, self.eps, residual=residual)
         return residual, out
 
-    def forward_rows(self, x, residual, rows):
+    def forward_rows(self, x, residual, rows, out_dtype=None):
+        if x is None:
+            # nothing waits to be added to the stream: the norm of its wanted rows alone
+            if residual is None or residual.dtype != torch.float32:
+                raise PartError("rms_norm: the norm of the stream's rows alone needs a 32-bit stream")
+            return K.rmsnorm_wide(None, self.weight, self.eps, residual=residual, rows=rows, out_dtype=out_dtype)
         if self.residual_float32 and residual is not None:
             return K.rmsnorm_wide(x, self.weight, self.eps, residual=residual, rows=rows)
         return K.rmsnorm(x, self.weight, self.eps, residual=residual, rows=rows)
+
+    def forward_branch(self, y, residual, copy_dtype=None):
+        """residual += norm(y), in 32-bit and in place: for a layer whose norm sits on the branch's output.  Returns
+        the new residual rounded to ``copy_dtype`` (None when that is 32-bit: the residual itself serves)."""
+        if residual.dtype != torch.float32:
+            raise PartError("rms_norm: a branch is normed and added to a 32-bit stream only")
+        return K.rmsnorm_branch(y, self.weight, self.eps, residual, copy_dtype)

@@ -7,6 +7,7 @@ f32(p) * inv_freq_j in 32-bit, cos and sin in 32-bit
 """
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import torch
@@ -44,16 +45,38 @@ class RotaryFrequencies(PositionEncoding):
     table and no longest position.  How the rotated dimensions are paired is the mixer's business."""
     GRAPH_SAFE_PORTIONS = True
 
-    def __init__(self, rotary_dim: int, theta: float):
+    def __init__(self, rotary_dim: int, theta: float, long_wave_factor: float = 0.0, long_wave_low: float = 1.0,
+                 long_wave_high: float = 1.0, long_wave_original: int = 0):
+        """``long_wave_factor`` > 0 slows the long wavelengths down, by wavelength l = 2 pi / f against a length
+        ``long_wave_original``: l < original / high keeps f; l > original / low takes f / factor; between them,
+        with s = (original / l - low) / (high - low), (1 - s) f / factor + s f.  0: the plain frequencies."""
         if rotary_dim <= 0 or rotary_dim % 2:
             raise PartError(f"rotary_frequencies: rotary width {rotary_dim} must be positive and even")
         if theta <= 0:
             raise PartError(f"rotary_frequencies: base {theta} must be positive")
         self.rotary_dim = int(rotary_dim)
         self.theta = float(theta)
+        self.long_wave_factor = float(long_wave_factor or 0.0)
+        self.long_wave_low, self.long_wave_high = float(long_wave_low), float(long_wave_high)
+        self.long_wave_original = float(long_wave_original)
+        if self.long_wave_factor < 0 or (self.long_wave_factor > 0 and not (
+                self.long_wave_original > 0 and self.long_wave_low > 0 and self.long_wave_high > self.long_wave_low)):
+            raise PartError(f"rotary_frequencies: long waves scaled by {long_wave_factor} need an original length > 0 "
+                            f"and 0 < low < high, got {long_wave_original}, {long_wave_low}, {long_wave_high}")
         self.inv_freq: Optional[torch.Tensor] = None
 
-    def prepare(self, device):
+    def frequencies(self) -> torch.Tensor:
+        """The frequencies in 64-bit, on the host."""
         d = self.rotary_dim
         i = torch.arange(0, d // 2, dtype=torch.float64)
-        self.inv_freq = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / d).to(torch.float32).to(device)
+        f = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / d)
+        if self.long_wave_factor > 0:
+            length = 2.0 * math.pi / f
+            orig, low, high = self.long_wave_original, self.long_wave_low, self.long_wave_high
+            s = (orig / length - low) / (high - low)
+            blended = (1.0 - s) * f / self.long_wave_factor + s * f
+            f = torch.where(length < orig / high, f, torch.where(length > orig / low, f / self.long_wave_factor, blended))
+        return f
+
+    def prepare(self, device):
+        self.inv_freq = self.frequencies().to(torch.float32).to(device)

@@ -18,12 +18,15 @@ from .engine.engine import Engine, StepEntry
 class TraceRunner:
     def __init__(self, model_dir: Optional[str], dtype: str, max_tokens: Optional[int] = None,
                  page_size: Optional[int] = None, device: str = "cuda:0", num_pages: Optional[int] = None,
-                 random_config: Optional[dict] = None, weights_seed: int = 0):
+                 random_config: Optional[dict] = None, weights_seed: int = 0, state_slots: Optional[int] = None):
         """``model_dir``: a folder with config.json and safetensors; or ``random_config`` (a config.json's
         content): that model with weights drawn on the device from ``weights_seed``.  The pool holds
         ``max_tokens`` tokens, or ``num_pages`` pages of ``page_size`` tokens: exactly what live requests may
-        hold, so pages are used again."""
+        hold, so pages are used again.  ``state_slots``: slots for per-request state of fixed size (models with
+        such mixers): as many as requests may be live at once, so slots are used again too."""
         cfg = EngineConfig(dtype=dtype, device=device)
+        if state_slots is not None:
+            cfg.max_state_slots = int(state_slots)
         if page_size is not None:
             cfg.page_size = int(page_size)
         if num_pages is not None:
