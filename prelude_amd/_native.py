@@ -87,10 +87,14 @@ _KERNEL_API = {
     "pa_moe_combine": (I, [P, I, P, P, P, F, P, P, P, I, I, I]),
     "pa_moe_route": (I, [P, P, I, P, P, P, P, I, I, I, F, I]),
     "pa_qknorm_rope_kv_freq": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I]),
+    "pa_attn_decode_sink": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, F, P, I, I]),
+    "pa_attn_prefill_sink": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P]),
     "pa_attn_generic_sink": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P]),
     "pa_rmsnorm_branch": (I, [P, I, P, P, I, c_long, P, P, P, I, I, F]),
     "pa_gated_rmsnorm": (I, [P, I, P, P, c_long, P, P, I, I, F]),
-    "pa_lightning_attn": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, I, I, I, I, I, I]),
+    "pa_lightning_attn": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I]),
+    "pa_lightning_attn_workspace": (c_long, [I, I, I, I, I, I]),
+    "pa_lightning_attn_chunked": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I]),
     "pa_argmax_scratch": (I, [I, I]),
     "pa_argmax": (I, [P, P, P, P, I, I]),
     "pa_argmax_static_capacity": (I, []),

@@ -134,6 +134,16 @@ int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc,
                     int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                     int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd, int page_size, int window,
                     float scale, float softcap);
+// pa_attn_decode and pa_attn_prefill with a sink per head (sink [nh], 32-bit, in the units of the scaled scores; null:
+// none): a head's softmax divides by sum_j exp(s_j) + exp(sink_h).
+int pa_attn_decode_sink(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                        int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                        float* workspace, int nseq, int nh, int nkv, int hd, int page_size, int window, float scale,
+                        float softcap, const float* sink, int split_keys, int max_splits);
+int pa_attn_prefill_sink(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                         int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
+                         int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd, int page_size, int window,
+                         float scale, float softcap, const float* sink);
 // min_prefix: the fewest keys any sequence has before its portion (0 if unknown), a hint for the cut of the work.
 // The same with the cut of the work given (for tests and measurements): tiles in pairs, heads a wavefront (1, 2, 4),
 // head groups a workgroup (1, 2), keys staged in LDS; -1 leaves one to the launcher.
@@ -198,7 +208,16 @@ int pa_gated_rmsnorm(void* stream, int dtype, const float* o, const void* gate, 
 // vdim] 32-bit; sequence s owns rows cu_q[s] .. cu_q[s + 1] and slot state_slots[s]; out [tokens, heads, vdim] 32-bit.
 int pa_lightning_attn(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off, const float* decay,
                       float* state, const int* state_slots, const int* cu_q, float* out, int nseq, int tokens, int heads,
-                      int dim, int vdim, int act);
+                      int dim, int vdim, int act, int max_len);
+// max_len > 0 above: sequences of more tokens are left alone, for the call below.  The sequences seq_ids[0 .. nlisted)
+// with more than `chunk` tokens (a multiple of 16 up to 256; at most max_len each) in chunks that the whole chip
+// works on at once: three passes (each chunk from a zero state, the states chained in order, what came before a chunk
+// added).  work: pa_lightning_attn_workspace(...) 32-bit words.
+long pa_lightning_attn_workspace(int nlisted, int tokens, int heads, int dim, int vdim, int chunk);
+int pa_lightning_attn_chunked(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off,
+                              const float* decay, float* state, const int* state_slots, const int* cu_q, const int* seq_ids,
+                              float* out, float* work, int nlisted, int tokens, int max_len, int heads, int dim, int vdim,
+                              int act, int chunk);
 
 // ---- attention through a latent (latent.hip) ----
 // in [tokens, q_rank + rank + rot]: cq_out [tokens, q_rank] = RMSNorm(first part) * wq; into the cache row slots[t]

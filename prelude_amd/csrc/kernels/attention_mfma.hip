@@ -52,9 +52,16 @@ struct ScoreMap {
   float c;        // exponent per unit of (bent) score
   float cap;      // 0: none
   float cap_in;   // scale / cap
+  // a sink per head (or null): one more term exp(sink[h]) of the softmax's denominator that brings no value, in the
+  // units of the scaled scores.  It joins when a row's sums are finished: against the reference exponent `ref` (the
+  // row's maximum times c, log2 domain) the term is 2^(sink log2(e) - ref).
+  const float* sink;
+  __device__ __forceinline__ float sink_term(int h, float ref) const {
+    return sink ? exp2f(sink[h] * kLog2e - ref) : 0.f;
+  }
 };
-__host__ inline ScoreMap score_map(float scale, float softcap) {
-  return softcap > 0.f ? ScoreMap{kLog2e, softcap, scale / softcap} : ScoreMap{scale * kLog2e, 0.f, 0.f};
+__host__ inline ScoreMap score_map(float scale, float softcap, const float* sink = nullptr) {
+  return softcap > 0.f ? ScoreMap{kLog2e, softcap, scale / softcap, sink} : ScoreMap{scale * kLog2e, 0.f, 0.f, sink};
 }
 
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
@@ -550,7 +557,7 @@ __global__ __launch_bounds__(WAVES* kWave, WAVES == 8 ? 1 : 3) void attn_decode_
     }
     const int h = kvh * group + qt * 16 + qi;
     if (nsplit == 1) {
-      out[(token * nh + h) * HD + d] = (bf16)(o / l);
+      out[(token * nh + h) * HD + d] = (bf16)(o / (l + c.sink_term(h, mm)));
     } else {
       const size_t slot = ((size_t)seq_idx * nh + h) * max_splits + split_idx;
       part_o[slot * HD + d] = o;
@@ -580,7 +587,7 @@ template <int HD>
 __global__ __launch_bounds__(merge_groups_of(HD) * ((HD + kWave - 1) / kWave * kWave)) void attn_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out, int nh, int window,
-    int split_keys, int max_splits) {
+    int split_keys, int max_splits, const float* __restrict__ sink) {
   constexpr int kBatch = 16;
   constexpr int TPG = (HD + kWave - 1) / kWave * kWave;   // threads a group
   __shared__ float group_acc[kMergeGroups][TPG];
@@ -629,8 +636,10 @@ __global__ __launch_bounds__(merge_groups_of(HD) * ((HD + kWave - 1) / kWave * k
       }
     }
   }
+  // a sink joins the finished sums once, against the same maximum as the splits
+  const float sink_l = sink ? exp2f(sink[h] * kLog2e - mm) : 0.f;
   if (groups == 1) {
-    if (col) out[(token * nh + h) * HD + d] = (bf16)(acc / l);
+    if (col) out[(token * nh + h) * HD + d] = (bf16)(acc / (l + sink_l));
     return;
   }
   group_acc[grp][d] = acc;
@@ -642,7 +651,7 @@ __global__ __launch_bounds__(merge_groups_of(HD) * ((HD + kWave - 1) / kWave * k
       a += group_acc[g][d];
       ll += group_l[g];
     }
-    out[(token * nh + h) * HD + d] = (bf16)(a / ll);
+    out[(token * nh + h) * HD + d] = (bf16)(a / (ll + sink_l));
   }
 }
 
@@ -689,7 +698,7 @@ __device__ __forceinline__ void prefill_tile(const bf16* __restrict__ q, bf16* _
   if (!qvalid) return;
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
-    const float inv = 1.0f / st[j].l[0];
+    const float inv = 1.0f / (st[j].l[0] + c.sink_term(head0 + j, st[j].reference()));
     bf16* orow = out + ((size_t)(row0 + t0 + r) * nh + head0 + j) * HD;
 #pragma unroll
     for (int t = 0; t < OT; ++t) {
@@ -925,7 +934,7 @@ __device__ __forceinline__ void prefill_tile_lds(StageLds<HD>& lds, const bf16* 
   if (!qvalid) return;
 #pragma unroll
   for (int j = 0; j < GT; ++j) {
-    const float inv = 1.0f / st[j].l[0];
+    const float inv = 1.0f / (st[j].l[0] + c.sink_term(head0 + j, st[j].reference()));
     bf16* orow = out + ((size_t)(row0 + t0 + r) * nh + head0 + j) * HD;
 #pragma unroll
     for (int t = 0; t < OT; ++t) {
@@ -976,7 +985,7 @@ template <int HD, bool FUSED>
 int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                   float* part_o, float* part_ml, int nseq, int nh, int nkv, int page_shift, int window, float scale,
-                  float softcap, int split_keys, int max_splits, const FusedQkv& fq) {
+                  float softcap, const float* sink, int split_keys, int max_splits, const FusedQkv& fq) {
   const int qtiles = (nh / nkv + 15) / 16;
   // Grids of 513 to 4,096 workgroups are dealt out so that each XCD gets a contiguous stretch of them; measured in
   // the decode step of a 4B model: batch 8 at 4,096 keys +0.9 %, batch 9 to 12 +0.8 to 1.2 %, and the kernel alone
@@ -1002,15 +1011,15 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
   if (eight_wavefronts) {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 8>), grid, dim3(8 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
-                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap), split_keys, max_splits, fq, contiguous);
+                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap, sink), split_keys, max_splits, fq, contiguous);
   } else if (two_wavefronts) {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 2>), grid, dim3(2 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
-                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap), split_keys, max_splits, fq, contiguous);
+                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap, sink), split_keys, max_splits, fq, contiguous);
   } else {
     hipLaunchKernelGGL((attn_decode_kernel<HD, FUSED, 4>), grid, dim3(4 * kWave), 0, st, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, part_o,
-                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap), split_keys, max_splits, fq, contiguous);
+                       part_ml, nh, nkv, page_shift, window, score_map(scale, softcap, sink), split_keys, max_splits, fq, contiguous);
   }
   if (int rc = check_launch("attn_decode")) return rc;
   if (max_splits > 1) {
@@ -1019,7 +1028,7 @@ int launch_decode(hipStream_t st, const void* q, const void* kc, const void* vc,
     const int groups = runs < merge_groups_of(HD) ? runs : merge_groups_of(HD);
     hipLaunchKernelGGL(attn_decode_merge_kernel<HD>, dim3(nh, nseq), dim3(groups * ((HD + kWave - 1) / kWave * kWave)),
                        0, st, part_o, part_ml, seq_ids, cu_q, context_lens, (bf16*)out, nh, window, split_keys,
-                       max_splits);
+                       max_splits, sink);
     return check_launch("attn_decode_merge");
   }
   return 0;
@@ -1029,7 +1038,7 @@ template <int HD, int GT, int HW>
 int launch_prefill_staged(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                           int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                           int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale,
-                          float softcap, int paired) {
+                          float softcap, const float* sink, int paired) {
   const int tiles = (max_q_len + 63) / 64;
   dim3 grid(nkv * (nh / nkv / (GT * HW)), paired == 1 ? (tiles + 1) / 2 : tiles, nseq);
   if (paired == 2) grid = dim3(grid.x, nseq, tiles);
@@ -1041,7 +1050,7 @@ int launch_prefill_staged(hipStream_t st, const void* q, const void* kc, const v
     return pa::fail("attn_prefill: %zu bytes of LDS refused: %s", sizeof(StageLds<HD>), hipGetErrorString(allowed));
   hipLaunchKernelGGL((attn_prefill_lds_kernel<HD, GT, HW>), grid, dim3(256 * HW), sizeof(StageLds<HD>), st,
                      (const bf16*)q, (const bf16*)kc, (const bf16*)vc, block_table, table_stride, seq_ids, cu_q,
-                     context_lens, (bf16*)out, nh, nkv, page_shift, window, score_map(scale, softcap), paired);
+                     context_lens, (bf16*)out, nh, nkv, page_shift, window, score_map(scale, softcap, sink), paired);
   return check_launch("attn_prefill");
 }
 
@@ -1049,20 +1058,20 @@ template <int HD, int GT>
 int launch_prefill_gt(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                       int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out,
                       int nseq, int max_q_len, int nh, int nkv, int page_shift, int window, float scale, float softcap,
-                      int paired, int hw, bool staged) {
+                      const float* sink, int paired, int hw, bool staged) {
   const int tiles = (max_q_len + 63) / 64;
   if (!staged && paired == 2) paired = 0;   // the kernel that reads the cache itself has the one order
   dim3 grid(nkv * (nh / nkv / GT), paired == 1 ? (tiles + 1) / 2 : tiles, nseq);
   if (staged) {
     if (hw == 2)
       return launch_prefill_staged<HD, GT, 2>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
-                                              nseq, max_q_len, nh, nkv, page_shift, window, scale, softcap, paired);
+                                              nseq, max_q_len, nh, nkv, page_shift, window, scale, softcap, sink, paired);
     return launch_prefill_staged<HD, GT, 1>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out,
-                                            nseq, max_q_len, nh, nkv, page_shift, window, scale, softcap, paired);
+                                            nseq, max_q_len, nh, nkv, page_shift, window, scale, softcap, sink, paired);
   }
   hipLaunchKernelGGL((attn_prefill_kernel<HD, GT>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kc,
                      (const bf16*)vc, block_table, table_stride, seq_ids, cu_q, context_lens, (bf16*)out, nh, nkv,
-                     page_shift, window, score_map(scale, softcap), paired);
+                     page_shift, window, score_map(scale, softcap, sink), paired);
   return check_launch("attn_prefill");
 }
 
@@ -1076,7 +1085,7 @@ template <int HD>
 int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc, const int* block_table,
                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens, void* out, int nseq,
                    int max_q_len, int min_prefix, int nh, int nkv, int page_shift, int window, float scale,
-                   float softcap, const PrefillCut& want) {
+                   float softcap, const float* sink, const PrefillCut& want) {
   const int group = nh / nkv;
   // How the work is cut: tiles in pairs (an early and a late tile of the causal triangle, so workgroups finish
   // together) and as many heads per wavefront as share the keys and fit the registers (wider heads would not fit
@@ -1213,7 +1222,7 @@ int launch_prefill(hipStream_t st, const void* q, const void* kc, const void* vc
   PA_REQUIRE(gt <= gt_most, "attn_prefill: %d heads a wavefront, head_dim %d takes up to %d", gt, HD, gt_most);
 #define PA_GT(GT)                                                                                                   \
   return launch_prefill_gt<HD, GT>(st, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, \
-                                   max_q_len, nh, nkv, page_shift, window, scale, softcap, paired, hw, staged)
+                                   max_q_len, nh, nkv, page_shift, window, scale, softcap, sink, paired, hw, staged)
   if constexpr (HD <= 64) {   // four heads' state of a wider head does not fit 256 registers: not built, never chosen
     if (gt == 4) PA_GT(4);
   }
@@ -1259,10 +1268,10 @@ extern "C" long pa_attn_decode_workspace(int nseq, int nh, int hd, int max_split
   return max_splits <= 1 ? 0 : (long)nseq * nh * max_splits * (hd + 2);
 }
 
-extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+static int attn_decode_entry(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                               int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                               void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
-                              int window, float scale, float softcap, int split_keys, int max_splits) {
+                              int window, float scale, float softcap, const float* sink, int split_keys, int max_splits) {
   if (nseq == 0) return 0;
   PA_REQUIRE(softcap >= 0.f, "attn_decode: a score cap of %g is negative (0 means none)", (double)softcap);
   if (int rc = check_common("attn_decode", nseq, nh, nkv, page_size, table_stride, window)) return rc;
@@ -1274,7 +1283,7 @@ extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const
 #define PA_CALL(HD)                                                                                                  \
   return launch_decode<HD, false>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q,         \
                                   context_lens, out, part_o, part_ml, nseq, nh, nkv, __builtin_ctz(page_size), window, \
-                                  scale, softcap, split_keys, max_splits, FusedQkv{})
+                                  scale, softcap, sink, split_keys, max_splits, FusedQkv{})
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }
@@ -1310,10 +1319,10 @@ extern "C" int pa_attn_decode_fused(void* stream, const void* qkv, const float* 
   const int shift = __builtin_ctz(page_size);
   if (hd == 64)
     return launch_decode<64, true>((hipStream_t)stream, nullptr, kc, vc, block_table, table_stride, seq_ids, cu_q,
-                                   context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, softcap,
+                                   context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, softcap, nullptr,
                                    split_keys, max_splits, fq);
   return launch_decode<128, true>((hipStream_t)stream, nullptr, kc, vc, block_table, table_stride, seq_ids, cu_q,
-                                  context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, softcap,
+                                  context_lens, out, part_o, part_ml, nseq, nh, nkv, shift, window, scale, softcap, nullptr,
                                   split_keys, max_splits, fq);
 }
 
@@ -1335,23 +1344,58 @@ extern "C" int pa_attn_prefill_cut(void* stream, const void* q, const void* kc, 
   cut.paired = paired, cut.heads = heads, cut.groups = groups, cut.staged = staged;
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, softcap, cut)
+                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, softcap, nullptr, cut)
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
 }
 
-extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+static int attn_prefill_entry(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
                                int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
                                void* out, int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd,
-                               int page_size, int window, float scale, float softcap) {
+                               int page_size, int window, float scale, float softcap, const float* sink) {
   if (nseq == 0) return 0;
   if (int rc = check_common("attn_prefill", nseq, nh, nkv, page_size, table_stride, window)) return rc;
   PA_REQUIRE(max_q_len >= 1 && min_prefix >= 0, "attn_prefill: longest portion %d, shortest prefix %d", max_q_len, min_prefix);
   PA_REQUIRE(softcap >= 0.f, "attn_prefill: a score cap of %g is negative (0 means none)", (double)softcap);
 #define PA_CALL(HD)                                                                                                   \
   return launch_prefill<HD>((hipStream_t)stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, \
-                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, softcap,  \
+                            out, nseq, max_q_len, min_prefix, nh, nkv, __builtin_ctz(page_size), window, scale, softcap, sink, \
                             PrefillCut{})
   PA_HD_SWITCH(hd, PA_CALL)
 #undef PA_CALL
+}
+
+extern "C" int pa_attn_decode(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                              int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                              void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
+                              int window, float scale, float softcap, int split_keys, int max_splits) {
+  return attn_decode_entry(stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, workspace, nseq, nh,
+                           nkv, hd, page_size, window, scale, softcap, nullptr, split_keys, max_splits);
+}
+
+extern "C" int pa_attn_prefill(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                               int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                               void* out, int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd,
+                               int page_size, int window, float scale, float softcap) {
+  return attn_prefill_entry(stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, max_q_len,
+                            min_prefix, nh, nkv, hd, page_size, window, scale, softcap, nullptr);
+}
+
+// The two with a sink per head (sink [nh], 32-bit, in the units of the scaled scores; null: none): a head's softmax
+// divides by sum_j exp(s_j) + exp(sink_h).  The term joins a row's finished sums (in decode: after the splits are merged).
+extern "C" int pa_attn_decode_sink(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                                   int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                                   void* out, float* workspace, int nseq, int nh, int nkv, int hd, int page_size,
+                                   int window, float scale, float softcap, const float* sink, int split_keys,
+                                   int max_splits) {
+  return attn_decode_entry(stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, workspace, nseq, nh,
+                           nkv, hd, page_size, window, scale, softcap, sink, split_keys, max_splits);
+}
+
+extern "C" int pa_attn_prefill_sink(void* stream, const void* q, const void* kc, const void* vc, const int* block_table,
+                                    int table_stride, const int* seq_ids, const int* cu_q, const int* context_lens,
+                                    void* out, int nseq, int max_q_len, int min_prefix, int nh, int nkv, int hd,
+                                    int page_size, int window, float scale, float softcap, const float* sink) {
+  return attn_prefill_entry(stream, q, kc, vc, block_table, table_stride, seq_ids, cu_q, context_lens, out, nseq, max_q_len,
+                            min_prefix, nh, nkv, hd, page_size, window, scale, softcap, sink);
 }

@@ -9,10 +9,21 @@
 // state slot state_slots[s]; a request's portions may be cut anywhere, the state carries over.
 //
 // pa_lightning_attn: the recurrence as it stands, on the vector ALU, for any sizes and both element types.  A
-// workgroup owns (64 value columns, head, sequence): four wavefronts split the rows of S between them (row d to
-// wavefront d % 4), each thread keeps its rows of one column in registers and walks the tokens in order, sixteen at
-// a time through LDS; the four partial dot products of a token are added in wavefront order.  The order of every sum
+// workgroup owns (64 value columns, head, sequence): four wavefronts split the rows of S between them (a quarter
+// each), each thread keeps its rows of one column in registers and walks the tokens in order, sixteen at a time
+// through LDS; the four partial dot products of a token are added in wavefront order.  The order of every sum
 // follows the token's place in its sequence alone, so a token's output is the same bits however its prompt was cut.
+//
+// pa_lightning_attn_chunked: the same sums for long portions with the whole chip at work.  A portion is cut into
+// chunks of C tokens; with S_b the state before a chunk and i a token's place in it,
+//
+//   o_i   = sum_{j <= i} a^(i-j) (q_i . k_j) v_j  +  a^(i+1) S_b^T q_i        (inside the chunk  +  from before it)
+//   S_b'  = a^n S_b + U,   U = sum_j a^(n-1-j) k_j v_j^T                      (n tokens in the chunk)
+//
+// so (1) every chunk runs the recurrence from a zero state on its own, which gives the first sum and U, (2) one pass
+// over the chunks of a sequence in order turns the U into the S_b and leaves the final state in the slot, (3) every
+// chunk adds the second term.  All three keep to 32-bit and to non-negative powers of a.  Sequences of at most one
+// chunk are left to pa_lightning_attn.
 #include "common.h"
 #include "api.h"
 
@@ -20,57 +31,107 @@ namespace pa {
 
 constexpr int kLaTokens = 16;    // tokens staged at a time
 constexpr int kLaCols = 64;      // value columns a workgroup
-constexpr int kLaParts = 4;      // wavefronts, each with a share of the state's rows
+constexpr int kLaParts = 4;      // wavefronts, each with a quarter of the state's rows
+constexpr int kLaMaxChunk = 256;
 
 __device__ __forceinline__ float la_act(float x, int act) { return act == 1 ? x / (1.0f + expf(-x)) : x; }
 
-// R: rows of the state a thread keeps (dim <= 4 R)
-template <typename T, int R>
+enum LaMode : int { kLaWhole = 0, kLaLocal = 1, kLaApply = 2 };
+
+// Where chunk j of the sequence that starts at packed row `row0` and is the z-th of the launch keeps its state: every
+// sequence adds at most one partial chunk, so floor(row0 / C) + z + j is different for every chunk of the launch and
+// below tokens / C + sequences.
+__device__ __forceinline__ size_t la_chunk_index(int row0, int chunk, int z, int j) { return (size_t)(row0 / chunk + z + j); }
+
+// R: rows of the state a thread keeps (dim <= 4 R, R a multiple of 4).
+// kLaWhole: grid (column tiles, heads, sequences); sequences longer than `max_len` tokens (> 0) are left alone.
+// kLaLocal / kLaApply: grid (column tiles, heads, listed sequences x max_chunks); sequences of at most one chunk and
+// chunks past a sequence's end leave at once.
+template <typename T, int R, int MODE>
 __global__ __launch_bounds__(kLaParts* kLaCols) void lightning_attn_kernel(
     const T* __restrict__ qkv, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
-    float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_q, float* __restrict__ out,
-    int heads, int dim, int vdim, int act) {
-  __shared__ float qs[kLaTokens][4 * R];
-  __shared__ float ks[kLaTokens][4 * R];
+    float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_q,
+    const int* __restrict__ seq_ids, float* __restrict__ out, float* __restrict__ work, int heads, int dim, int vdim, int act,
+    int max_len, int chunk, int max_chunks) {
+  __shared__ __align__(16) float qs[kLaTokens][4 * R];
+  __shared__ __align__(16) float ks[kLaTokens][4 * R];
   __shared__ float vs[kLaTokens][kLaCols];
   __shared__ float part[kLaParts][kLaTokens][kLaCols];
+  __shared__ float pw[MODE == kLaApply ? kLaMaxChunk : 1];
   const int col = threadIdx.x % kLaCols, w = threadIdx.x / kLaCols;
-  const int c0 = blockIdx.x * kLaCols, h = blockIdx.y, seq = blockIdx.z;
-  const int row0 = cu_q[seq], row1 = cu_q[seq + 1];
+  const int c0 = blockIdx.x * kLaCols, h = blockIdx.y;
+  int seq, z = 0, j = 0;
+  if (MODE == kLaWhole) {
+    seq = blockIdx.z;
+  } else {
+    z = blockIdx.z / max_chunks, j = blockIdx.z % max_chunks;
+    seq = seq_ids[z];
+  }
+  int row0 = cu_q[seq], row1 = cu_q[seq + 1];
   const int slot = state_slots[seq];
   if (slot < 0 || row1 <= row0) return;   // the same for the whole workgroup
+  if (MODE == kLaWhole && max_len > 0 && row1 - row0 > max_len) return;
+  float* sp;
+  if (MODE == kLaWhole) {
+    sp = state + (((size_t)slot * heads + h) * dim) * vdim + c0 + col;
+  } else {
+    if (row1 - row0 <= chunk || row0 + j * chunk >= row1) return;
+    sp = work + ((la_chunk_index(row0, chunk, z, j) * heads + h) * dim) * vdim + c0 + col;
+    row0 += j * chunk;
+    row1 = row1 < row0 + chunk ? row1 : row0 + chunk;
+  }
   const bool live = c0 + col < vdim;
   const float a = decay[h];
-  float* sp = state + (((size_t)slot * heads + h) * dim) * vdim + c0 + col;
+  if (MODE == kLaApply) {
+    for (int i = threadIdx.x; i < chunk; i += kLaParts * kLaCols) pw[i] = powf(a, (float)(i + 1));
+  }
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int d = r * kLaParts + w;
-    S[r] = (live && d < dim) ? sp[(size_t)d * vdim] : 0.f;
+    const int d = w * R + r;
+    S[r] = (MODE != kLaLocal && live && d < dim) ? sp[(size_t)d * vdim] : 0.f;
   }
   for (int t0 = row0; t0 < row1; t0 += kLaTokens) {
     const int n = row1 - t0 < kLaTokens ? row1 - t0 : kLaTokens;
     __syncthreads();   // the block before has been read
-    for (int i = threadIdx.x; i < n * dim; i += kLaParts * kLaCols) {
-      const int t = i / dim, d = i % dim;
-      const T* src = qkv + (size_t)(t0 + t) * ld + (size_t)h * dim + d;
-      qs[t][d] = la_act(to_f32(src[q_off]), act);
-      ks[t][d] = la_act(to_f32(src[k_off]), act);
+    for (int i = threadIdx.x; i < n * 4 * R; i += kLaParts * kLaCols) {
+      const int t = i / (4 * R), d = i % (4 * R);
+      float qv = 0.f, kv = 0.f;   // rows past dim are zeros: they leave the sums alone
+      if (d < dim) {
+        const T* src = qkv + (size_t)(t0 + t) * ld + (size_t)h * dim + d;
+        qv = la_act(to_f32(src[q_off]), act);
+        if (MODE != kLaApply) kv = la_act(to_f32(src[k_off]), act);
+      }
+      qs[t][d] = qv;
+      if (MODE != kLaApply) ks[t][d] = kv;
     }
-    for (int i = threadIdx.x; i < n * kLaCols; i += kLaParts * kLaCols) {
-      const int t = i / kLaCols, c = i % kLaCols;
-      vs[t][c] = c0 + c < vdim ? la_act(to_f32(qkv[(size_t)(t0 + t) * ld + v_off + (size_t)h * vdim + c0 + c]), act) : 0.f;
+    if (MODE != kLaApply) {
+      for (int i = threadIdx.x; i < n * kLaCols; i += kLaParts * kLaCols) {
+        const int t = i / kLaCols, c = i % kLaCols;
+        vs[t][c] = c0 + c < vdim ? la_act(to_f32(qkv[(size_t)(t0 + t) * ld + v_off + (size_t)h * vdim + c0 + c]), act) : 0.f;
+      }
     }
     __syncthreads();
     for (int t = 0; t < n; ++t) {
-      const float v = vs[t][col];
       float acc = 0.f;
+      if (MODE == kLaApply) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int d = r * kLaParts + w;
-        if (d < dim) {
-          S[r] = fmaf(a, S[r], ks[t][d] * v);
-          acc = fmaf(S[r], qs[t][d], acc);
+        for (int r = 0; r < R; r += 4) {
+          const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[t][w * R + r]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc = fmaf(S[r + e], q4[e], acc);
+        }
+      } else {
+        const float v = vs[t][col];
+#pragma unroll
+        for (int r = 0; r < R; r += 4) {
+          const f32x4 k4 = *reinterpret_cast<const f32x4*>(&ks[t][w * R + r]);
+          const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[t][w * R + r]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            S[r + e] = fmaf(a, S[r + e], k4[e] * v);
+            acc = fmaf(S[r + e], q4[e], acc);
+          }
         }
       }
       part[w][t][col] = acc;
@@ -78,32 +139,74 @@ __global__ __launch_bounds__(kLaParts* kLaCols) void lightning_attn_kernel(
     __syncthreads();
     for (int i = threadIdx.x; i < n * kLaCols; i += kLaParts * kLaCols) {
       const int t = i / kLaCols, c = i % kLaCols;
-      if (c0 + c < vdim)
-        out[((size_t)(t0 + t) * heads + h) * vdim + c0 + c] = ((part[0][t][c] + part[1][t][c]) + part[2][t][c]) + part[3][t][c];
+      if (c0 + c < vdim) {
+        const float sum = ((part[0][t][c] + part[1][t][c]) + part[2][t][c]) + part[3][t][c];
+        float* o = out + ((size_t)(t0 + t) * heads + h) * vdim + c0 + c;
+        if (MODE == kLaApply) *o += pw[t0 + t - row0] * sum;
+        else *o = sum;
+      }
     }
   }
-  if (live) {
+  if (MODE != kLaApply && live) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int d = r * kLaParts + w;
+      const int d = w * R + r;
       if (d < dim) sp[(size_t)d * vdim] = S[r];
     }
   }
 }
 
-template <typename T>
-static int launch_lightning(hipStream_t st, const T* qkv, long ld, int q_off, int k_off, int v_off, const float* decay,
-                            float* state, const int* state_slots, const int* cu_q, float* out, int nseq, int heads, int dim,
-                            int vdim, int act) {
-  dim3 grid((vdim + kLaCols - 1) / kLaCols, heads, nseq);
-#define PA_LA(R)                                                                                                        \
-  hipLaunchKernelGGL((lightning_attn_kernel<T, R>), grid, dim3(kLaParts* kLaCols), 0, st, qkv, ld, q_off, k_off, v_off, \
-                     decay, state, state_slots, cu_q, out, heads, dim, vdim, act)
+// The chunks of one listed sequence in order: work[chunk] holds U coming in and the state before the chunk going
+// out; the state slot gives the start and receives the end.  A thread an element of a head's state.
+__global__ __launch_bounds__(256) void lightning_scan_kernel(const float* __restrict__ decay, float* __restrict__ state,
+                                                            const int* __restrict__ state_slots, const int* __restrict__ cu_q,
+                                                            const int* __restrict__ seq_ids, float* __restrict__ work,
+                                                            int heads, int per_head, int chunk) {
+  const int z = blockIdx.z, h = blockIdx.y;
+  const int seq = seq_ids[z];
+  const int row0 = cu_q[seq], len = cu_q[seq + 1] - row0;
+  const int slot = state_slots[seq];
+  if (slot < 0 || len <= chunk) return;
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= per_head) return;
+  const float a = decay[h];
+  const float a_chunk = powf(a, (float)chunk);
+  float* sp = state + ((size_t)slot * heads + h) * per_head + e;
+  float S = *sp;
+  const int chunks = (len + chunk - 1) / chunk;
+  for (int j = 0; j < chunks; ++j) {
+    float* wp = work + (la_chunk_index(row0, chunk, z, j) * heads + h) * per_head + e;
+    const float U = *wp;
+    *wp = S;
+    const int n = len - j * chunk;
+    S = fmaf(n >= chunk ? a_chunk : powf(a, (float)n), S, U);
+  }
+  *sp = S;
+}
+
+template <typename T, int MODE>
+static void launch_lightning(hipStream_t st, dim3 grid, const T* qkv, long ld, int q_off, int k_off, int v_off,
+                             const float* decay, float* state, const int* state_slots, const int* cu_q, const int* seq_ids,
+                             float* out, float* work, int heads, int dim, int vdim, int act, int max_len, int chunk,
+                             int max_chunks) {
+#define PA_LA(R)                                                                                                          \
+  hipLaunchKernelGGL((lightning_attn_kernel<T, R, MODE>), grid, dim3(kLaParts* kLaCols), 0, st, qkv, ld, q_off, k_off,     \
+                     v_off, decay, state, state_slots, cu_q, seq_ids, out, work, heads, dim, vdim, act, max_len, chunk, max_chunks)
   if (dim <= 32) PA_LA(8);
   else if (dim <= 64) PA_LA(16);
   else if (dim <= 128) PA_LA(32);
   else PA_LA(64);
 #undef PA_LA
+}
+
+static int lightning_check(const char* what, int nseq, int tokens, int heads, int dim, int vdim, long ld, int q_off, int k_off,
+                           int v_off, int act) {
+  PA_REQUIRE(nseq > 0 && tokens > 0 && heads > 0 && vdim > 0, "%s: bad sizes seqs=%d tokens=%d heads=%d vdim=%d", what, nseq,
+             tokens, heads, vdim);
+  PA_REQUIRE(dim > 0 && dim <= 256, "%s: a key width of %d is outside 1..256", what, dim);
+  PA_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && ld >= (long)heads * dim, "%s: bad offsets or row stride %ld", what, ld);
+  PA_REQUIRE(act == 0 || act == 1, "%s: unknown activation code %d", what, act);
+  PA_REQUIRE(heads <= 65535, "%s: %d heads exceed the grid", what, heads);
   return 0;
 }
 
@@ -111,24 +214,66 @@ static int launch_lightning(hipStream_t st, const T* qkv, long ld, int q_off, in
 
 using namespace pa;
 
+// max_len > 0: sequences of more tokens are left alone (they go to pa_lightning_attn_chunked).
 extern "C" int pa_lightning_attn(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off,
                                  const float* decay, float* state, const int* state_slots, const int* cu_q, float* out,
-                                 int nseq, int tokens, int heads, int dim, int vdim, int act) {
+                                 int nseq, int tokens, int heads, int dim, int vdim, int act, int max_len) {
   if (nseq == 0 || tokens == 0) return 0;
-  PA_REQUIRE(nseq > 0 && tokens > 0 && heads > 0 && vdim > 0, "lightning_attn: bad sizes seqs=%d tokens=%d heads=%d vdim=%d", nseq,
-             tokens, heads, vdim);
-  PA_REQUIRE(dim > 0 && dim <= 256, "lightning_attn: a key width of %d is outside 1..256", dim);
-  PA_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && ld >= (long)heads * dim, "lightning_attn: bad offsets or row stride %ld", ld);
-  PA_REQUIRE(act == 0 || act == 1, "lightning_attn: unknown activation code %d", act);
-  PA_REQUIRE(nseq <= 65535 && heads <= 65535, "lightning_attn: %d sequences x %d heads exceed the grid", nseq, heads);
+  if (int rc = lightning_check("lightning_attn", nseq, tokens, heads, dim, vdim, ld, q_off, k_off, v_off, act)) return rc;
+  PA_REQUIRE(nseq <= 65535, "lightning_attn: %d sequences exceed the grid", nseq);
   hipStream_t st = (hipStream_t)stream;
+  dim3 grid((vdim + kLaCols - 1) / kLaCols, heads, nseq);
   if (dtype == kF32)
-    launch_lightning<float>(st, (const float*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q, out, nseq, heads, dim,
-                            vdim, act);
+    launch_lightning<float, kLaWhole>(st, grid, (const float*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
+                                      nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1);
   else if (dtype == kBF16)
-    launch_lightning<bf16>(st, (const bf16*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q, out, nseq, heads, dim,
-                           vdim, act);
+    launch_lightning<bf16, kLaWhole>(st, grid, (const bf16*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
+                                     nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1);
   else
     return pa::fail("lightning_attn: unknown element type code %d", dtype);
   return check_launch("lightning_attn");
+}
+
+// 32-bit words of workspace for the listed sequences' chunk states
+extern "C" long pa_lightning_attn_workspace(int nlisted, int tokens, int heads, int dim, int vdim, int chunk) {
+  if (chunk <= 0) return 0;
+  return ((long)tokens / chunk + nlisted) * heads * dim * vdim;
+}
+
+// The sequences seq_ids[0 .. nlisted) that have more than `chunk` tokens (at most max_len each), in chunks.
+extern "C" int pa_lightning_attn_chunked(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off,
+                                         const float* decay, float* state, const int* state_slots, const int* cu_q,
+                                         const int* seq_ids, float* out, float* work, int nlisted, int tokens, int max_len,
+                                         int heads, int dim, int vdim, int act, int chunk) {
+  if (nlisted == 0 || tokens == 0 || max_len <= chunk) return 0;
+  if (int rc = lightning_check("lightning_attn_chunked", nlisted, tokens, heads, dim, vdim, ld, q_off, k_off, v_off, act)) return rc;
+  PA_REQUIRE(chunk >= kLaTokens && chunk % kLaTokens == 0 && chunk <= kLaMaxChunk,
+             "lightning_attn_chunked: chunks of %d tokens are not a multiple of %d up to %d", chunk, kLaTokens, kLaMaxChunk);
+  PA_REQUIRE(seq_ids && work, "lightning_attn_chunked: no list of sequences or no workspace");
+  const int max_chunks = (max_len + chunk - 1) / chunk;
+  PA_REQUIRE((long)nlisted * max_chunks <= 65535, "lightning_attn_chunked: %d sequences x %d chunks exceed the grid", nlisted, max_chunks);
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((vdim + kLaCols - 1) / kLaCols, heads, nlisted * max_chunks);
+  const int per_head = dim * vdim;
+  dim3 scan_grid((per_head + 255) / 256, heads, nlisted);
+#define PA_LA_PASS(T, MODE)                                                                                               \
+  launch_lightning<T, MODE>(st, grid, (const T*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q, seq_ids, out, \
+                            work, heads, dim, vdim, act, 0, chunk, max_chunks)
+#define PA_LA_SCAN()                                                                                                      \
+  hipLaunchKernelGGL(lightning_scan_kernel, scan_grid, dim3(256), 0, st, decay, state, state_slots, cu_q, seq_ids, work,   \
+                     heads, per_head, chunk)
+  if (dtype == kF32) {
+    PA_LA_PASS(float, kLaLocal);
+    PA_LA_SCAN();
+    PA_LA_PASS(float, kLaApply);
+  } else if (dtype == kBF16) {
+    PA_LA_PASS(bf16, kLaLocal);
+    PA_LA_SCAN();
+    PA_LA_PASS(bf16, kLaApply);
+  } else {
+    return pa::fail("lightning_attn_chunked: unknown element type code %d", dtype);
+  }
+#undef PA_LA_PASS
+#undef PA_LA_SCAN
+  return check_launch("lightning_attn_chunked");
 }

@@ -825,10 +825,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         raise NativeError("attention: index arrays do not match the number of tokens")
     out = torch.empty_like(q)
     if sink is not None:
-        _dev(sink)
-        _f32(sink, "sinks")
-        if tuple(sink.shape) != (nh,):
-            raise NativeError(f"attention: sinks {tuple(sink.shape)} for {nh} heads")
+        _check_sinks(sink, nh)
         check(kernels().pa_attn_generic_sink(_stream(), _code(q), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
                                              block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out), t, nh,
                                              k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale),
@@ -890,7 +887,8 @@ def mfma_attention_supported(head_dim: int, page_size: int) -> bool:
 
 
 def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_context: int,
-                     window: int, scale: float, every_seq: bool = False, softcap: float = 0.0) -> None:
+                     window: int, scale: float, every_seq: bool = False, softcap: float = 0.0,
+                     sink: Optional[torch.Tensor] = None) -> None:
     """Matrix-core attention for the sequences ``seq_ids`` (each feeding one token); writes their rows of ``out``.
     ``every_seq``: ``seq_ids`` is 0, 1, .. (a step of single tokens only); the kernels then count for themselves
     instead of reading it, which is one trip to memory less before their first key."""
@@ -903,11 +901,26 @@ def attention_decode(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_le
     max_splits = _decode_splits(max_context, window, k_cache.shape[2])
     words = kernels().pa_attn_decode_workspace(n, nh, hd, max_splits)
     ws = torch.empty((max(words, 1),), dtype=torch.float32, device=q.device)
+    if sink is not None:
+        _check_sinks(sink, nh)
+        check(kernels().pa_attn_decode_sink(_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+                                            block_table.shape[1], None if every_seq else _ptr(seq_ids), _ptr(cu_q),
+                                            _ptr(context_lens), _ptr(out), _ptr(ws), n, nh, k_cache.shape[1], hd,
+                                            k_cache.shape[2], int(window), float(scale), float(softcap), _ptr(sink),
+                                            DECODE_SPLIT_KEYS, max_splits))
+        return
     check(kernels().pa_attn_decode(_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
                                    block_table.shape[1], None if every_seq else _ptr(seq_ids), _ptr(cu_q),
                                    _ptr(context_lens), _ptr(out),
                                    _ptr(ws), n, nh, k_cache.shape[1], hd, k_cache.shape[2], int(window), float(scale),
                                    float(softcap), DECODE_SPLIT_KEYS, max_splits))
+
+
+def _check_sinks(sink: torch.Tensor, heads: int) -> None:
+    _dev(sink)
+    _f32(sink, "sinks")
+    if tuple(sink.shape) != (heads,):
+        raise NativeError(f"attention: sinks {tuple(sink.shape)} for {heads} heads")
 
 
 def attention_decode_fused_supported(nh: int, nkv: int, hd: int, rot: int, page_size: int) -> bool:
@@ -951,7 +964,8 @@ def attention_decode_fused(qkv, q_weight, k_weight, cos, sin, slots, eps: float,
 
 
 def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_lens, out, max_q_len: int,
-                      window: int, scale: float, cut=None, min_prefix: int = 0, softcap: float = 0.0) -> None:
+                      window: int, scale: float, cut=None, min_prefix: int = 0, softcap: float = 0.0,
+                      sink: Optional[torch.Tensor] = None) -> None:
     """Matrix-core attention for the sequences ``seq_ids`` (portions of several tokens); writes their rows of ``out``.
 
     ``min_prefix`` is the fewest keys any of the sequences has before its portion: a hint for how the launcher
@@ -967,7 +981,12 @@ def attention_prefill(q, k_cache, v_cache, block_table, seq_ids, cu_q, context_l
     args = (_stream(), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_ids),
             _ptr(cu_q), _ptr(context_lens), _ptr(out), n, int(max_q_len), int(min_prefix), nh, k_cache.shape[1], hd,
             k_cache.shape[2], int(window), float(scale), float(softcap))
-    if cut is None:
+    if sink is not None:
+        if cut is not None:
+            raise NativeError("attention_prefill: a given cut and a sink do not go together")
+        _check_sinks(sink, nh)
+        check(kernels().pa_attn_prefill_sink(*args, _ptr(sink)))
+    elif cut is None:
         check(kernels().pa_attn_prefill(*args))
     else:
         check(kernels().pa_attn_prefill_cut(*args, *(int(c) for c in cut)))
@@ -982,16 +1001,17 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
     tokens go to the split decode kernel, portions to the prefill kernel.
     Everything else (float32, other sizes) goes to the generic kernel.
     """
-    if q.dtype == torch.bfloat16 and step.decode_seqs is not None and sink is None \
+    if q.dtype == torch.bfloat16 and step.decode_seqs is not None \
             and mfma_attention_supported(q.shape[2], k_cache.shape[2]):
         out = torch.empty_like(q)
         if step.n_decode:
             attention_decode(q, k_cache, v_cache, group.block_table, step.decode_seqs, step.cu_q, step.context_lens,
                              out, step.max_decode_context, window, scale,
-                             every_seq=step.n_prefill == 0 and step.n_decode == step.num_seqs, softcap=softcap)
+                             every_seq=step.n_prefill == 0 and step.n_decode == step.num_seqs, softcap=softcap, sink=sink)
         if step.n_prefill:
             attention_prefill(q, k_cache, v_cache, group.block_table, step.prefill_seqs, step.cu_q, step.context_lens,
-                              out, step.max_prefill_q, window, scale, min_prefix=step.min_prefill_prefix, softcap=softcap)
+                              out, step.max_prefill_q, window, scale, min_prefix=step.min_prefill_prefix, softcap=softcap,
+                              sink=sink)
         return out
     return attention_generic(q, k_cache, v_cache, group.block_table, step.seq_of_token, step.positions, window, scale,
                              softcap, sink)
