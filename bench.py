@@ -89,6 +89,37 @@ def libodra_record(args):
     return out
 
 
+# ``--arch fazopel``: a decoder of the Fazopel design at layer sizes of a real model of that kind: three layers of
+# linear attention with a decaying state to one of grouped-query attention (keys for values, a sink in the softmax);
+# the first layer's feed-forward dense, the others routed experts with a gated shared one -- beside the same Qwen3
+# decoder as above (same width, depth and vocabulary)
+def fazopel_shape(layers=12, width=2048, vocab=65536):
+    heads = 16
+    lightning = dict(heads=heads, dim=128, vdim=128, decay=[1.0 - 2.0 ** -(5.0 + 3.0 * h / heads) for h in range(heads)])
+    attention = dict(heads=16, kv_heads=8, dim=128, vdim=128, scale=128 ** -0.5,
+                     rot=dict(base=1000000.0, dims=64, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+    dense = dict(kind="dense", ff=8192)
+    moe = dict(kind="moe", expert=dict(ff=1408, limit=7.0), router=dict(experts=64, top=6, scale=2.5), shared=dict(ff=2816, limit=7.0))
+    return dict(architecture="Fazopel", vocab=vocab, width=width, norm=dict(eps=1e-6),
+                layers=[dict(type="attention" if i % 4 == 3 else "lightning", mixer=attention if i % 4 == 3 else lightning,
+                             mlp=dense if i == 0 else moe) for i in range(layers)])
+
+
+def fazopel_record(args):
+    """Prefill and decode throughput of the Fazopel shape and of the Qwen3 shape beside it, same points."""
+    out = {"arch": "fazopel", "dtype": args.dtype, "layers": args.layers or 12, "points": {}}
+    for name, raw in (("fazopel", fazopel_shape(args.layers or 12)), ("qwen3_beside", qwen3_beside_libodra(args.layers or 12))):
+        pts = {}
+        for t in (512, args.prefill_tokens):
+            sec = time_prefill(raw, args.dtype, t, reps=3)
+            pts[f"prefill_{t}"] = {"ms": round(sec * 1e3, 3), "tok_per_s": round(t / sec, 1)}
+        for b, ctx in ((1, args.context), (args.batch, args.context), (32, args.context)):
+            sec = decode_point(raw, args.dtype, b, ctx, max(8, args.steps // 2), max(2, args.warmup // 2), None)
+            pts[f"decode_b{b}_ctx{ctx}"] = {"ms": round(sec * 1e3, 3), "tok_per_s": round(b / sec, 1)}
+        out["points"][name] = pts
+    return out
+
+
 def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
     """The engine in its random-weights mode: the product's own loader, tensors drawn on the device."""
     from prelude_amd.config import EngineConfig
@@ -324,8 +355,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 0.6B, 8B or 32B")
-    ap.add_argument("--arch", default="qwen3", choices=["qwen3", "libodra"],
-                    help="libodra: prefill and decode of the Libodra design at a real model's layer sizes beside a Qwen3 "
+    ap.add_argument("--arch", default="qwen3", choices=["qwen3", "libodra", "fazopel"],
+                    help="libodra, fazopel: prefill and decode of that design at a real model's layer sizes beside a Qwen3 "
                          "decoder of equal size, as one record (the default run and its record are Qwen3's)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the points at other batches and lengths")
@@ -351,6 +382,9 @@ def main() -> int:
     import torch
     if args.arch == "libodra":
         print(json.dumps(libodra_record(args)), flush=True)
+        return 0
+    if args.arch == "fazopel":
+        print(json.dumps(fazopel_record(args)), flush=True)
         return 0
     raw = dict(SHAPES[args.shape])
     name = f"Qwen3-{args.shape.upper()} shape"

@@ -1163,14 +1163,22 @@ def gated_rmsnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps
 LIGHTNING_ACTIVATIONS = {None: 0, "none": 0, "silu": 1}
 
 
+LIGHTNING_CHUNK = 128      # tokens a chunk of the chunked form; portions of more tokens go to it (bfloat16 engine)
+
+
 def lightning_attention(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, state: torch.Tensor,
-                        step, heads: int, dim: int, vdim: int, activation: Optional[str] = "silu") -> torch.Tensor:
+                        step, heads: int, dim: int, vdim: int, activation: Optional[str] = "silu",
+                        chunk: Optional[int] = None) -> torch.Tensor:
     """Linear attention with a decaying state: per head S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t.
 
     qkv [T, width]: a token's queries [heads, dim], keys [heads, dim] and values [heads, vdim] start at columns
     ``q_off``, ``k_off``, ``v_off`` and pass through ``activation``; decay float32 [heads]; state float32
     [slots, heads, dim, vdim], read and left by the step's sequences through ``step.state_slots``.  Returns
-    float32 [T, heads, vdim]."""
+    float32 [T, heads, vdim].
+
+    ``chunk``: portions of more tokens are cut into chunks of that many that run side by side (three passes; the
+    sums are the same up to rounding, in another order); 0: every sequence token by token, whose sums do not depend
+    on how a prompt was cut.  None: ``LIGHTNING_CHUNK`` for a bfloat16 engine, 0 for a 32-bit one."""
     _dev(qkv, decay, state)
     _f32(decay, "decays")
     _f32(state, "state")
@@ -1181,10 +1189,20 @@ def lightning_attention(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, d
                           f"for {heads} heads of {dim} and {vdim}")
     if activation not in LIGHTNING_ACTIVATIONS:
         raise NativeError(f"lightning_attention: activation {activation!r} is not one of {sorted(map(str, LIGHTNING_ACTIVATIONS))}")
+    if chunk is None:
+        chunk = LIGHTNING_CHUNK if qkv.dtype == torch.bfloat16 else 0
+    chunked = chunk > 0 and step.n_prefill > 0 and step.max_prefill_q > chunk
     out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qkv.device)
-    check(kernels().pa_lightning_attn(_stream(), _code(qkv), _ptr(qkv), qkv.shape[1], int(q_off), int(k_off), int(v_off),
-                                      _ptr(decay), _ptr(state), _ptr(step.state_slots), _ptr(step.cu_q), _ptr(out),
-                                      step.num_seqs, t, heads, dim, vdim, LIGHTNING_ACTIVATIONS[activation]))
+    args = (_code(qkv), _ptr(qkv), qkv.shape[1], int(q_off), int(k_off), int(v_off), _ptr(decay), _ptr(state),
+            _ptr(step.state_slots), _ptr(step.cu_q))
+    act = LIGHTNING_ACTIVATIONS[activation]
+    check(kernels().pa_lightning_attn(_stream(), *args, _ptr(out), step.num_seqs, t, heads, dim, vdim, act,
+                                      int(chunk) if chunked else 0))
+    if chunked:
+        words = kernels().pa_lightning_attn_workspace(step.n_prefill, t, heads, dim, vdim, int(chunk))
+        work = torch.empty((max(words, 1),), dtype=torch.float32, device=qkv.device)
+        check(kernels().pa_lightning_attn_chunked(_stream(), *args, _ptr(step.prefill_seqs), _ptr(out), _ptr(work),
+                                                  step.n_prefill, t, int(step.max_prefill_q), heads, dim, vdim, act, int(chunk)))
     return out
 
 

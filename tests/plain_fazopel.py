@@ -158,3 +158,105 @@ def forward(cfg, w, tokens, dtype=torch.float64, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return (unit_rms(x, eps) * w["final.norm"]) @ w["head"].T
+
+
+# ---- configurations and weights of the tests' own --------------------------------------------------------------------
+def _lightning(heads, dim, vdim, decay):
+    return {"type": "lightning", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": list(decay)}}
+
+
+def _attention(heads, kv_heads, dim, scale, base, dims, scaling=None):
+    rot = {"base": base, "dims": dims}
+    if scaling is not None:
+        rot["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
+    return {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale, "rot": rot}}
+
+
+def _moe(experts, top, ff, limit, scale, shared=None):
+    f = {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top, "scale": scale}}
+    if shared is not None:
+        f["shared"] = {"ff": shared[0], "limit": shared[1]}
+    return f
+
+
+def tiny_config_p():
+    """Three heads of unequal decay, a layer run twice, a layer without a feed-forward, heads of 32 and 16."""
+    first = dict(_lightning(3, 16, 24, (0.5, 0.9, 0.995)), mlp=_moe(5, 2, 24, 1.5, 1.5, shared=(40, 0.7)))
+    return {"architecture": "Fazopel", "vocab": 97, "width": 64, "norm": {"eps": 1e-5}, "layers": [
+        first,
+        dict(_attention(4, 2, 32, 0.2, 1000.0, 16, scaling=(8.0, 1.0, 4.0, 64)), mlp={"kind": "dense", "ff": 96}),
+        dict(first, weights_of=0),
+        dict(_attention(6, 3, 16, 0.3, 10000.0, 16), mlp=None)]}
+
+
+def tiny_config_q():
+    """Attention first; one KV head under four query heads; odd state sizes; a decay of 1; experts without a shared one."""
+    first = dict(_attention(4, 1, 64, 0.11, 50000.0, 32, scaling=(4.0, 1.0, 2.0, 128)), mlp=_moe(8, 3, 16, 2.0, 1.0))
+    return {"architecture": "Fazopel", "vocab": 211, "width": 128, "norm": {"eps": 1e-6}, "layers": [
+        first,
+        dict(_lightning(2, 40, 72, (0.97, 1.0)), mlp={"kind": "dense", "ff": 160}),
+        dict(first, weights_of=0),
+        dict(_lightning(4, 32, 32, (0.6, 0.8, 0.9, 0.99)), mlp=_moe(4, 1, 32, 0.8, 2.5, shared=(24, 1.2)))]}
+
+
+def tiny_config_r():
+    """Ones: one head, one KV head, every expert chosen, a decay of 0; a head size the matrix cores do not take; the
+    whole head rotated; value columns beyond two tiles."""
+    return {"architecture": "Fazopel", "vocab": 61, "width": 48, "norm": {"eps": 1e-5}, "layers": [
+        dict(_lightning(1, 8, 130, (0.9,)), mlp=_moe(3, 3, 8, 1.0, 1.0, shared=(8, 1.0))),
+        dict(_attention(1, 1, 24, 0.25, 100.0, 24), mlp={"kind": "dense", "ff": 40}),
+        dict(_lightning(2, 8, 8, (0.0, 0.75)), mlp=None)]}
+
+
+def tensor_shapes(cfg):
+    """name -> shape of every tensor a model of this configuration stores."""
+    h, out = cfg["width"], {"embed": (cfg["vocab"], cfg["width"]), "final.norm": (cfg["width"],), "head": (cfg["vocab"], cfg["width"])}
+    for i, lc in enumerate(cfg["layers"]):
+        if "weights_of" in lc:
+            continue
+        p, m = f"l{i}.", lc["mixer"]
+        out[p + "norm1"] = (h,)
+        if lc["type"] == "lightning":
+            qk, vv = m["heads"] * m["dim"], m["heads"] * m["vdim"]
+            out.update({p + "mix.q": (qk, h), p + "mix.k": (qk, h), p + "mix.v": (vv, h), p + "mix.g": (vv, h),
+                        p + "mix.o": (h, vv), p + "mix.norm": (vv,)})
+        else:
+            out.update({p + "mix.q": (m["heads"] * m["dim"], h), p + "mix.k": (m["kv_heads"] * m["dim"], h),
+                        p + "mix.q.norm": (m["dim"],), p + "mix.k.norm": (m["dim"],), p + "mix.o": (h, m["heads"] * m["dim"])})
+        f = lc.get("mlp")
+        if f is None:
+            continue
+        out[p + "norm2"] = (h,)
+        if f["kind"] == "dense":
+            out.update({p + "mlp.up": (f["ff"], h), p + "mlp.down": (h, f["ff"])})
+            continue
+        e = f["router"]["experts"]
+        out.update({p + "mlp.router": (e, h), p + "mlp.correction": (e,)})
+        for j in range(e):
+            ff = f["expert"]["ff"]
+            out.update({f"{p}mlp.e{j}.gate": (ff, h), f"{p}mlp.e{j}.up": (ff, h), f"{p}mlp.e{j}.down": (h, ff)})
+        if f.get("shared"):
+            ff = f["shared"]["ff"]
+            out.update({p + "mlp.shared.gate": (ff, h), p + "mlp.shared.up": (ff, h), p + "mlp.shared.down": (h, ff),
+                        p + "mlp.shared.sg": (1, h)})
+    return out
+
+
+def random_weights(cfg, seed):
+    """Weights as a file would hold them: values of bfloat16, here as float32.  Matrices ~ N(0, 1 / in) (the gates'
+    and the experts' a little larger, so that clamps bite), norm weights around one, corrections of the size of the
+    scores' differences."""
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for name, shape in tensor_shapes(cfg).items():
+        if len(shape) == 1 and name.endswith(("norm1", "norm2", ".norm")):
+            t = 1.0 + 0.2 * torch.randn(shape, generator=g)
+        elif name.endswith("correction"):
+            t = 0.2 * torch.randn(shape, generator=g)
+        elif name == "embed":
+            t = torch.randn(shape, generator=g)
+        else:
+            boost = 2.0 if (".mlp.e" in name or ".shared." in name or name.endswith("router")) else 1.0
+            t = torch.randn(shape, generator=g) * boost / math.sqrt(shape[-1])
+        w[name] = t.to(torch.bfloat16).to(torch.float32)
+    return w

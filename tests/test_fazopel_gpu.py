@@ -1,0 +1,555 @@
+"""Fazopel on the GPU against the plain implementation (``plain_fazopel``): every mechanism's kernels alone, then the
+engine under schedules (whole, token by token, portions down to two tokens, unequal requests in one batch, pages and
+state slots used again, long decoding) and greedy generation through ``LLM``.  Configurations and weights are the
+tests' own.
+
+The 32-bit engine is held to the plain implementation at every row, with routers that choose.  In bfloat16 a
+router's choice between two experts whose scores nearly agree can fall the other way than in 64-bit, which is no
+fault and moves that token's logits, and those of the tokens behind it, by as much as their spread: no bound tells
+that from a fault.  So under the bfloat16 engine the same configurations run with every expert chosen (``top`` =
+``experts``: router, weights, grouped products and the sum are all there, only the choice is not), every row is held
+to a quarter of the spread and nine rows in ten to a tenth (``mostly``); the choice itself is tested in bfloat16
+where the router sees the very same numbers as the plain one (the part alone, below)."""
+import functools
+import json
+import math
+import os
+import tempfile
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import plain_fazopel as pf
+from helpers import check
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+TD = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+_keep = []
+
+
+def close(got, want, dtype, what, scale=None):
+    got, want = got.double().cpu(), want.double()
+    bound = (2e-5 if dtype == "float32" else 2e-2) * (float(want.abs().max()) if scale is None else scale)
+    err = float((got - want).abs().max())
+    assert err <= bound, f"{what}: {err:.3e} > {bound:.3e}"
+
+
+def mostly(got, ref, dtype, what):
+    """Every row against the plain logits: 32-bit to rounding; bfloat16 to a quarter of the spread everywhere and to a
+    tenth at nine rows in ten (the narrowest of the tests' models is 48 wide, where single rows reach 0.15)."""
+    if dtype == "float32":
+        return check(got, ref, dtype, what)
+    got = torch.as_tensor(got).double().reshape(ref.shape)
+    err = (got - ref).abs().reshape(len(ref), -1).max(dim=1).values / float(ref.double().std())
+    assert float(err.max()) <= 0.25, f"{what}: row {int(err.argmax())} is off by {float(err.max()):.3f} of the spread"
+    over = int((err > 0.1).sum())
+    assert over <= max(1, len(err) // 10), f"{what}: {over} of {len(err)} rows are off by more than a tenth of the spread"
+
+
+def rnd(shape, seed, dtype, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(TD[dtype])
+
+
+# ---- norms -----------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [48, 256, 1000, 2560, 9000])
+def test_a_branch_is_normed_and_added_to_the_stream(gpu, dtype, hidden):
+    from prelude_amd.ops import kernels as K
+    y = rnd((7, hidden), 1, dtype, 3.0)
+    res = torch.randn((7, hidden), generator=torch.Generator().manual_seed(2)) * 3
+    w = 1 + 0.3 * torch.randn(hidden, generator=torch.Generator().manual_seed(3))
+    want = res.double() + pf.unit_rms(y.double(), 1e-5) * w.double()
+    r = res.to(gpu)
+    copy = K.rmsnorm_branch(y.to(gpu), w.to(gpu), 1e-5, r, TD[dtype])
+    close(r, want, "float32", "the stream keeps the unrounded sum")
+    if dtype == "float32":
+        assert copy is None
+    else:
+        assert torch.equal(copy, r.to(torch.bfloat16)), "the copy is the new stream, rounded once"
+    parts = torch.randn((3, 7, hidden), generator=torch.Generator().manual_seed(4))
+    r2 = res.to(gpu)
+    K.rmsnorm_branch(K.SliceSums(parts.to(gpu), TD[dtype]), w.to(gpu), 1e-5, r2, TD[dtype])
+    close(r2, res.double() + pf.unit_rms(parts.double().sum(0), 1e-5) * w.double(), "float32", "from partial sums")
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=gpu)
+    out = K.rmsnorm_wide(None, w.to(gpu), 1e-5, residual=r, rows=rows, out_dtype=TD[dtype])
+    close(out, (pf.unit_rms(want, 1e-5) * w.double())[[5, 0, 5]], dtype, "the norm of the stream's rows alone")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [24, 144, 260, 2048])
+def test_unit_rms_scaled_and_gated(gpu, dtype, width):
+    from prelude_amd.ops import kernels as K
+    o = torch.randn((9, width), generator=torch.Generator().manual_seed(5)) * 4
+    wide = rnd((9, 3 * width + 8), 6, dtype, 2.0)          # the gate lies inside a wider projection
+    w = 1 + 0.3 * torch.randn(width, generator=torch.Generator().manual_seed(7))
+    gate = wide[:, width + 8: 2 * width + 8]
+    want = pf.unit_rms(o.double(), 1e-6) * w.double() * torch.sigmoid(gate.double())
+    got = K.gated_rmsnorm(o.to(gpu), wide.to(gpu)[:, width + 8: 2 * width + 8], w.to(gpu), 1e-6)
+    assert got.dtype == TD[dtype]
+    close(got, want, dtype, "gated norm")
+
+
+# ---- the recurrent mixer's kernel ---------------------------------------------------------------------------------
+def _step_of(lengths, slots, gpu):
+    """What the recurrence reads of a step: packed rows, slots, and the sequences of more than one token."""
+    cu = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    pre = [i for i, n in enumerate(lengths) if n > 1]
+    return types.SimpleNamespace(
+        num_seqs=len(lengths), cu_q=torch.tensor(cu, device=gpu), state_slots=torch.tensor(slots, dtype=torch.int32, device=gpu),
+        prefill_seqs=torch.tensor(pre, dtype=torch.int32, device=gpu), n_prefill=len(pre),
+        max_prefill_q=max([lengths[i] for i in pre], default=0))
+
+
+def _plain_recurrence(q, k, v, a, S):
+    """o_t = S_t^T q_t with S_t = a S_(t-1) + k_t v_t^T for one head; q, k [n, d], v [n, vd]; returns (o, S)."""
+    out = torch.zeros(q.shape[0], v.shape[1], dtype=torch.float64)
+    for t in range(q.shape[0]):
+        S = a * S + k[t][:, None] * v[t][None, :]
+        out[t] = S.T @ q[t]
+    return out, S
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chunk", [0, 16, 48])
+@pytest.mark.parametrize("H,d,vd,decay", [(3, 16, 24, (0.5, 0.9, 0.995)), (2, 40, 72, (0.97, 1.0)), (1, 8, 130, (0.0,)),
+                                          (2, 128, 128, (0.999, 0.7)), (1, 256, 64, (0.9,))])
+def test_the_recurrence_alone(gpu, dtype, chunk, H, d, vd, decay):
+    """Unequal sequences in one launch (single tokens, portions that end inside, at and just past a chunk's edge),
+    each from a state of its own in a slot of its own; outputs and the states left behind."""
+    from prelude_amd.ops import kernels as K
+    lengths = [1, 47, 48, 49, 1, 2, 113, 16, 17]
+    slots = [7, 2, 9, 0, 4, 11, 5, 1, 8]
+    T = sum(lengths)
+    width = 2 * H * d + H * vd + 5                           # five columns of something else in front
+    x = rnd((T, width), 11, dtype, 1.2)
+    state0 = torch.randn((12, H, d, vd), generator=torch.Generator().manual_seed(12))
+    state = state0.to(gpu)
+    step = _step_of(lengths, slots, gpu)
+    dec = torch.tensor(decay, dtype=torch.float32)
+    out = K.lightning_attention(x.to(gpu), 5, 5 + H * d, 5 + 2 * H * d, dec.to(gpu), state, step, H, d, vd, "silu", chunk=chunk)
+    assert out.dtype == torch.float32 and state.dtype == torch.float32
+    xs = pf.silu(x.double())
+    row = 0
+    scale = None
+    for n, slot in zip(lengths, slots):
+        for h in range(H):
+            q = xs[row:row + n, 5 + h * d: 5 + (h + 1) * d]
+            k = xs[row:row + n, 5 + H * d + h * d: 5 + H * d + (h + 1) * d]
+            v = xs[row:row + n, 5 + 2 * H * d + h * vd: 5 + 2 * H * d + (h + 1) * vd]
+            o, S = _plain_recurrence(q, k, v, float(dec[h].double()), state0[slot, h].double())
+            close(out[row:row + n, h], o, "float32", f"outputs of a sequence of {n}, head {h}", scale=float(o.abs().max()) * 5)
+            close(state[slot, h], S, "float32", f"state after a sequence of {n}, head {h}", scale=float(S.abs().max()) * 5)
+        row += n
+    untouched = [s for s in range(12) if s not in slots]
+    assert torch.equal(state[untouched].cpu(), state0[untouched]), "slots of no sequence are left alone"
+
+
+def test_the_recurrence_does_not_depend_on_the_cut_in_32_bit(gpu):
+    """Token by token, in portions and whole: the same bits, since every sum follows the token's place alone."""
+    from prelude_amd.ops import kernels as K
+    H, d, vd, n = 2, 24, 40, 75
+    x = rnd((n, 2 * H * d + H * vd), 13, "float32")
+    dec = torch.tensor([0.9, 0.99], device=gpu)
+    outs = []
+    for cuts in ([n], [1] * n, [7, 2, 30, 1, 35]):
+        state = torch.zeros((1, H, d, vd), device=gpu)
+        got, row = [], 0
+        for c in cuts:
+            got.append(K.lightning_attention(x[row:row + c].to(gpu), 0, H * d, 2 * H * d, dec, state, _step_of([c], [0], gpu), H, d, vd))
+            row += c
+        outs.append((torch.cat(got).cpu(), state.cpu()))
+    for o, s in outs[1:]:
+        assert torch.equal(o, outs[0][0]) and torch.equal(s, outs[0][1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chunk", [0, 32])
+def test_a_token_far_back_shows_through_the_state(gpu, dtype, chunk):
+    """One early token whose key and value stand out, 700 tokens back, through a decay near one: the last outputs are
+    made of it (and of nothing, under the head whose decay forgets it)."""
+    from prelude_amd.ops import kernels as K
+    H, d, vd, n = 2, 16, 16, 704
+    x = rnd((n, 2 * H * d + H * vd), 14, dtype, 0.05)
+    x[:, :H * d] = 1.0                                     # every query sees every row of the state
+    x[3, H * d: 2 * H * d] = 6.0                           # token 3: a large key ...
+    x[3, 2 * H * d:] = 6.0                                 # ... and a large value, in both heads
+    dec = torch.tensor([0.999, 0.9])
+    state = torch.zeros((1, H, d, vd), device=gpu)
+    out = K.lightning_attention(x.to(gpu), 0, H * d, 2 * H * d, dec.to(gpu), state, _step_of([n], [0], gpu), H, d, vd, "silu", chunk=chunk)
+    xs = pf.silu(x.double())
+    for h in range(H):
+        o, _ = _plain_recurrence(xs[:, h * d:(h + 1) * d], xs[:, H * d + h * d: H * d + (h + 1) * d],
+                                 xs[:, 2 * H * d + h * vd: 2 * H * d + (h + 1) * vd], float(dec[h].double()), torch.zeros(d, vd, dtype=torch.float64))
+        close(out[-8:, h], o[-8:], "float32", f"head {h}", scale=float(o[-8:].abs().max()) * 5)
+    far = float(out[-1, 0].abs().mean()), float(out[-1, 1].abs().mean())
+    assert far[0] > 20 * far[1], "the slow head still holds token 3, the fast one has let it go"
+
+
+# ---- attention: rotation from frequencies, keys for values, a sink ------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,rot", [(4, 2, 32, 16), (6, 3, 16, 16), (1, 1, 24, 24), (4, 1, 64, 32), (8, 2, 96, 48), (2, 2, 128, 0)])
+def test_rotation_from_frequencies_with_the_keys_cached_as_values(gpu, dtype, nh, nkv, hd, rot):
+    from prelude_amd.ops import kernels as K
+    T, page, pages, eps = 9, 8, 5, 1e-5
+    x = rnd((T, (nh + nkv) * hd), 21, dtype, 2.0)
+    qw, kw = 1 + 0.3 * torch.randn(hd), 1 + 0.3 * torch.randn(hd)
+    pos = torch.tensor([0, 1, 2, 63, 64, 1000, 7, 8, 65537], dtype=torch.int32)
+    slots = torch.randperm(page * pages)[:T].to(torch.int32)
+    rotc = {"base": 5000.0, "dims": rot, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 256}}
+    freq = pf.scaled_frequencies(rotc).to(torch.float32) if rot else None
+    kc = torch.zeros((pages, nkv, page, hd), dtype=TD[dtype], device=gpu)
+    vc = torch.zeros((pages, nkv, hd, page), dtype=TD[dtype], device=gpu)
+    q = K.qknorm_rope_kv(x.to(gpu), qw.to(gpu), kw.to(gpu), None, None, pos.to(gpu), slots.to(gpu), kc, vc, nh, nkv, hd, rot, eps,
+                         inv_freq=None if freq is None else freq.to(gpu), values_from_keys=True)
+    xd = x.double().reshape(T, nh + nkv, hd)
+    turn = (lambda t: pf.turn_halves(t, pos, freq.double())) if rot else (lambda t: t)
+    # angles of large positions: the 32-bit product p * f decides, hence the wider 32-bit bound
+    wide = float(xd.abs().max()) * (50 if dtype == "float32" else 1)
+    close(q, turn(pf.unit_rms(xd[:, :nh], eps) * qw.double()), dtype, "queries", scale=wide)
+    sl = slots.long()
+    got_k = kc.cpu()[sl // page, :, sl % page]                    # [T, nkv, hd]
+    got_v = vc.cpu()[sl // page, :, :, sl % page]                 # [T, nkv, hd]
+    close(got_k, turn(pf.unit_rms(xd[:, nh:], eps) * kw.double()), dtype, "cached keys", scale=wide)
+    assert torch.equal(got_v, x.reshape(T, nh + nkv, hd)[:, nh:]), "the cached values are the keys as projected"
+
+
+def _paged_kv(keys, vals, page, gpu, dtype, seed=0):
+    """Scatter sequences' keys and values [n_i, nkv, hd] over shuffled pages; stale pages hold rubbish."""
+    need = [-(-len(x) // page) for x in keys]
+    total = sum(need) + 3
+    perm = torch.randperm(total, generator=torch.Generator().manual_seed(seed)).tolist()
+    nkv, hd = keys[0].shape[1:]
+    kc = torch.full((total, nkv, page, hd), 55.0, dtype=TD[dtype])
+    vc = torch.full((total, nkv, hd, page), -55.0, dtype=TD[dtype])
+    table = torch.full((len(keys), max(need)), -1, dtype=torch.int32)
+    at = 0
+    for s, (k, v) in enumerate(zip(keys, vals)):
+        for j in range(need[s]):
+            p = perm[at]
+            at += 1
+            table[s, j] = p
+            n = min(page, len(k) - j * page)
+            kc[p, :, :n] = k[j * page: j * page + n].transpose(0, 1)
+            vc[p, :, :, :n] = v[j * page: j * page + n].permute(1, 2, 0)
+    return kc.to(gpu), vc.to(gpu), table.to(gpu)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sink", ["zero", "learned", None])
+@pytest.mark.parametrize("nh,nkv,hd,page", [(4, 2, 32, 8), (6, 3, 16, 16), (1, 1, 24, 4), (4, 1, 64, 16), (8, 2, 96, 16)])
+def test_attention_with_a_sink(gpu, dtype, sink, nh, nkv, hd, page):
+    """Portions and single tokens in one step over shuffled pages: a first token alone (its weight is
+    e^s / (1 + e^s), not 1), a portion from position 0, a portion far into its context whose first query looks
+    back at one key that stands out among hundreds, single tokens at contexts of one key, one page, and many."""
+    from prelude_amd.ops import kernels as K
+    from prelude_amd.engine.batch import GroupStep
+    ctx = [1, 45, 700, 1, page, 650, 2]        # keys after the step
+    qn = [1, 45, 52, 1, 1, 1, 2]               # tokens this step
+    g = torch.Generator().manual_seed(31)
+    keys = [(torch.randn((c, nkv, hd), generator=g) * 0.9).to(TD[dtype]) for c in ctx]
+    vals = [(torch.randn((c, nkv, hd), generator=g)).to(TD[dtype]) for c in ctx]
+    qs = [(torch.randn((n, nh, hd), generator=g) * 0.9).to(TD[dtype]) for n in qn]
+    keys[2][5] *= 4.0                          # a key far back that the portion's queries find
+    keys[5][page] *= 4.0                       # ... and one at a page's first place for a single token
+    scale = 0.9 / math.sqrt(hd)
+    sinks = None if sink is None else (torch.zeros(nh) if sink == "zero" else torch.randn(nh, generator=g) * 2)
+    kc, vc, table = _paged_kv(keys, vals, page, gpu, dtype, seed=3)
+    cu = np.concatenate([[0], np.cumsum(qn)]).astype(np.int32)
+    pos = np.concatenate([np.arange(c - n, c) for c, n in zip(ctx, qn)]).astype(np.int32)
+    seq = np.concatenate([[i] * n for i, n in enumerate(qn)]).astype(np.int32)
+    dec = [i for i, n in enumerate(qn) if n == 1]
+    pre = [i for i, n in enumerate(qn) if n > 1]
+    dev = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
+    step = types.SimpleNamespace(
+        positions=dev(pos), seq_of_token=dev(seq), cu_q=dev(cu), context_lens=dev(ctx), decode_seqs=dev(dec), prefill_seqs=dev(pre),
+        n_decode=len(dec), n_prefill=len(pre), num_seqs=len(ctx), max_decode_context=max(ctx[i] for i in dec),
+        max_prefill_q=max(qn[i] for i in pre), min_prefill_prefix=min(ctx[i] - qn[i] for i in pre))
+    out = K.attention(torch.cat(qs).to(gpu), kc, vc, GroupStep(table, None), step, 0, scale,
+                      sink=None if sinks is None else sinks.to(gpu))
+    row = 0
+    for s, (c, n) in enumerate(zip(ctx, qn)):
+        k, v, q = keys[s].double(), vals[s].double(), qs[s].double()
+        for h in range(nh):
+            kv = h // (nh // nkv)
+            sc = (q[:, h] @ k[:, kv].T) * scale
+            sc = sc.masked_fill(torch.arange(c)[None, :] > torch.arange(c - n, c)[:, None], -math.inf)
+            if sinks is None:
+                p = torch.softmax(sc, dim=-1)
+            else:
+                m = torch.maximum(sc.max(dim=-1, keepdim=True).values, sinks[h].double())
+                e = torch.exp(sc - m)
+                p = e / (e.sum(dim=-1, keepdim=True) + torch.exp(sinks[h].double() - m))
+            close(out[row:row + n, h], p @ v[:, kv], dtype, f"sequence {s} (context {c}, {n} tokens), head {h}",
+                  scale=float(v.abs().max()))
+        row += n
+
+
+# ---- experts -------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("E,top,T", [(5, 2, 40), (8, 3, 7), (3, 3, 19), (4, 1, 300), (70, 6, 33), (130, 8, 5)])
+def test_the_router_alone(gpu, E, top, T):
+    from prelude_amd.ops import kernels as K
+    g = torch.Generator().manual_seed(41)
+    logits = torch.randn((T, E + 2), generator=g) * 2          # one more column for a gate, and one nobody reads
+    corr = torch.randn(E, generator=g) * 0.1
+    choice, weights, gate = K.moe_route(logits.to(gpu), E, top, 1.7, corr.to(gpu), gate_col=E)
+    s = torch.softmax(logits[:, :E].double(), dim=-1)
+    want = torch.topk(s + corr.double(), top, dim=-1).indices
+    assert torch.equal(choice.cpu().reshape(T, top).long().sort(dim=1).values, want.sort(dim=1).values)
+    ws = torch.gather(s, 1, choice.cpu().reshape(T, top).long())
+    close(weights.reshape(T, top), ws / (ws.sum(dim=1, keepdim=True) + 1e-20) * 1.7, "float32", "weights")
+    close(gate, torch.sigmoid(logits[:, E].double()), "float32", "the shared expert's gate")
+    plain = K.moe_route(logits[:, :E].contiguous().to(gpu), E, top, 1.0)
+    assert plain[2] is None
+    assert torch.equal(plain[0].cpu().reshape(T, top).long().sort(dim=1).values, torch.topk(s, top, dim=-1).indices.sort(dim=1).values)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("E,top,T,ff,shared", [(5, 2, 50, 24, 40), (8, 3, 1, 16, 0), (3, 3, 33, 8, 8), (4, 1, 300, 32, 24), (12, 4, 400, 64, 128)])
+def test_routed_experts(gpu, dtype, E, top, T, ff, shared):
+    """The part alone on the numbers the plain one gets (so both routers see the same scores): unequal loads, an
+    expert nobody chooses, every expert chosen, one token, more tokens than a tile."""
+    from prelude_amd.parts import build_part
+    h = 64
+    f = pf._moe(E, top, ff, 0.9, 1.6, shared=(shared, 0.6) if shared else None)
+    cfg = {"vocab": 8, "width": h, "layers": [dict(pf._lightning(1, 8, 8, (0.5,)), mlp=f)]}
+    w = {k[len("l0.mlp."):]: v for k, v in pf.random_weights(cfg, 42).items() if k.startswith("l0.mlp.")}
+    if E >= 5:
+        w["correction"][E - 1] = -5.0                             # the last expert is never chosen
+    x = rnd((T, h), 43, dtype, 1.5)
+    part = build_part("ffn", "routed_experts", dict(hidden_size=h, num_experts=E, top=top, expert_size=ff, limit=0.9,
+                                                    route_scale=1.6, shared_size=shared, shared_limit=0.6))
+    dev = {}
+    for name, req in part.tensors().items():
+        t = w[name]
+        dev[name] = (t.to(TD[dtype]) if req.kind == "matrix" else t.float()).to(gpu)
+    part.load(dev, TD[dtype], gpu)
+    got = part.forward(x.to(gpu))
+    want = pf.routed_experts_ff(x.double(), {"m." + k: v.double() for k, v in w.items()}, "m.", f)
+    close(got, want, dtype, "routed experts", scale=float(want.abs().max()) * (1 if dtype == "float32" else 1.5))
+
+
+# ---- the engine under schedules -----------------------------------------------------------------------------------
+def every_expert_chosen(make):
+    def made():
+        cfg = make()
+        for lc in cfg["layers"]:
+            if lc.get("mlp") and lc["mlp"]["kind"] == "moe":
+                lc["mlp"]["router"]["top"] = lc["mlp"]["router"]["experts"]
+        return cfg
+    return made
+
+
+# (configuration, seed, page size); "pA", "qA", "rA": the same with every expert chosen, for the bfloat16 engine
+CONFIGS = {"p": (pf.tiny_config_p, 11, 8), "q": (pf.tiny_config_q, 12, 16), "r": (pf.tiny_config_r, 13, 4)}
+CONFIGS.update({k + "A": (every_expert_chosen(make), seed, page) for k, (make, seed, page) in list(CONFIGS.items())})
+
+
+def model_for(name, dtype):
+    return name if dtype == "float32" else name + "A"
+
+
+@functools.lru_cache(maxsize=None)
+def folder(name):
+    from prelude_amd.weights import write_safetensors
+    make, seed, _ = CONFIGS[name]
+    cfg = make()
+    w = pf.random_weights(cfg, seed)
+    tmp = tempfile.TemporaryDirectory(prefix=f"prelude_amd_fazopel_{name}_")
+    _keep.append(tmp)
+    with open(os.path.join(tmp.name, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(os.path.join(tmp.name, "model.safetensors"), {k: v.to(torch.bfloat16) for k, v in w.items()})
+    return tmp.name, cfg, w
+
+
+@functools.lru_cache(maxsize=None)
+def plain_logits(name, seed, length):
+    _, cfg, w = folder(name)
+    toks = torch.randint(0, cfg["vocab"], (length,), generator=torch.Generator().manual_seed(700 + seed)).tolist()
+    return toks, pf.forward(cfg, w, toks)
+
+
+def runner(name, dtype, max_tokens, **kw):
+    from prelude_amd.trace import TraceRunner
+    return TraceRunner(folder(name)[0], dtype, max_tokens, page_size=CONFIGS[name][2], **kw)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["p", "q", "r"])
+def test_whole_prompt_every_position(gpu, name, dtype):
+    name = model_for(name, dtype)
+    toks, ref = plain_logits(name, 0, 300)          # longer than two chunks of the recurrence's chunked form
+    r = runner(name, dtype, 512, state_slots=2)
+    got = r.step([{"id": "x", "tokens": toks, "want": list(range(len(toks)))}], ["x"])
+    mostly(got, ref, dtype, f"{name} whole")
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+
+
+def test_every_layer_of_the_stream(gpu):
+    """The stream after every run of a layer (a layer run twice counts twice), in 32-bit, against the plain one's."""
+    toks, _ = plain_logits("p", 0, 300)
+    _, cfg, w = folder("p")
+    want = []
+    pf.forward(cfg, w, toks[:40], layers_out=want)
+    r = runner("p", "float32", 64, state_slots=1)
+    seen = []
+    for b in r.engine.model.blocks:
+        def wrapped(*a, _f=b.forward, **k):
+            h, res = _f(*a, **k)
+            seen.append(res.clone())
+            return h, res
+        b.forward = wrapped
+    r.step([{"id": "x", "tokens": toks[:40], "want": [39]}], ["x"])
+    assert len(seen) == len(want) == len(cfg["layers"])
+    for i, (a, b) in enumerate(zip(seen, want)):
+        close(a, b, "float32", f"after layer run {i}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["p", "q", "r"])
+def test_prefill_then_token_by_token(gpu, name, dtype):
+    name = model_for(name, dtype)
+    toks, ref = plain_logits(name, 1, 140)
+    r = runner(name, dtype, 256, state_slots=1)
+    n = 40
+    outs = [r.step([{"id": 0, "tokens": toks[:n], "want": list(range(n))}])]
+    for i in range(n, len(toks)):          # a hundred single tokens: page borders, and in bfloat16 replays of a captured step
+        outs.append(r.step([{"id": 0, "tokens": [toks[i]], "want": [0]}]))
+    mostly(np.concatenate(outs), ref, dtype, f"{name} decode")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["p", "q", "r"])
+def test_from_the_first_token_one_by_one(gpu, name, dtype):
+    name = model_for(name, dtype)
+    toks, ref = plain_logits(name, 2, 40)
+    r = runner(name, dtype, 64, state_slots=1)
+    outs = [r.step([{"id": 0, "tokens": [t], "want": [0]}]) for t in toks]
+    mostly(np.concatenate(outs), ref, dtype, f"{name} one by one")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["p", "q", "r"])
+def test_portions_of_changing_size(gpu, name, dtype):
+    name = model_for(name, dtype)
+    toks, ref = plain_logits(name, 3, 420)
+    sizes = [7, 2, 13, 2, 1, 31, 2, 9, 16, 3, 8, 2, 64, 5, 129, 2, 128]
+    r = runner(name, dtype, 512, state_slots=1)
+    outs, i, k = [], 0, 0
+    while i < len(toks):
+        n = min(sizes[k % len(sizes)], len(toks) - i)
+        k += 1
+        outs.append(r.step([{"id": "p", "tokens": toks[i:i + n], "want": list(range(n))}]))
+        i += n
+    mostly(np.concatenate(outs), ref, dtype, f"{name} portions")
+
+
+def test_the_32_bit_logits_do_not_depend_on_the_cut(gpu):
+    """Whole, token by token and in portions: in 32-bit the logits agree far inside the bound against the plain ones."""
+    toks, _ = plain_logits("p", 4, 70)
+    runs = []
+    for cuts in ([70], [1] * 70, [5, 2, 40, 1, 22]):
+        r = runner("p", "float32", 128, state_slots=1)
+        outs, i = [], 0
+        for c in cuts:
+            outs.append(r.step([{"id": "c", "tokens": toks[i:i + c], "want": list(range(c))}]))
+            i += c
+        runs.append(np.concatenate(outs))
+    for other in runs[1:]:
+        assert float(np.abs(other - runs[0]).max()) <= 2e-6 * float(np.abs(runs[0]).max())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["p", "q", "r"])
+def test_unequal_requests_in_one_batch_with_pages_and_slots_used_again(gpu, name, dtype):
+    """Six requests of unequal length through a pool that holds three of them and three state slots: portions of
+    some beside single tokens of others; a request ends as soon as it is fed, and its pages and its slot (with the
+    state it left there) go to the next."""
+    name = model_for(name, dtype)
+    lengths = [90, 17, 64, 33, 200, 5]
+    seqs = [plain_logits(name, 10 + i, n) for i, n in enumerate(lengths)]
+    r = runner(name, dtype, 3 * 256, state_slots=3)
+    rng = np.random.default_rng(7)
+    fed, waiting, live = [0] * len(seqs), list(range(len(seqs))), []
+    got = [[] for _ in seqs]
+    while waiting or live:
+        while waiting and len(live) < 3:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for i in live:
+            left = lengths[i] - fed[i]
+            n = 1 if (fed[i] > 0 and rng.random() < 0.5) else int(min(left, rng.choice([2, 3, 16, 29, 40, 150])))
+            entries.append({"id": f"r{i}", "tokens": seqs[i][0][fed[i]:fed[i] + n], "want": list(range(n))})
+            fed[i] += n
+            if fed[i] == lengths[i]:
+                end.append(f"r{i}")
+        out = r.step(entries, end)
+        k = 0
+        for e in entries:
+            i = int(e["id"][1:])
+            got[i].append(out[k:k + len(e["tokens"])])
+            k += len(e["tokens"])
+        live = [i for i in live if fed[i] < lengths[i]]
+    for i, (toks, ref) in enumerate(seqs):
+        mostly(np.concatenate(got[i]), ref, dtype, f"{name} request {i}")
+    assert r.engine.tables.audit() == "" and r.engine.tables.num_requests() == 0
+    assert r.engine.tables.free_state_slots() == 3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_token_far_back_moves_the_last_logits(gpu, dtype):
+    """Hundreds of keys and a state hundreds of steps old: the engine follows the plain implementation when one
+    early token changes, and that change is one the bound would not let pass."""
+    name = model_for("q", dtype)
+    toks, ref = plain_logits(name, 20, 600)
+    _, cfg, w = folder(name)
+    other = list(toks)
+    other[3] = (toks[3] + 1) % cfg["vocab"]
+    ref2 = pf.forward(cfg, w, other)
+    assert float((ref[-10:] - ref2[-10:]).abs().max()) > 0.3 * float(ref.std()), "the change shows in the plain logits"
+    r = runner(name, dtype, 1280, state_slots=2)
+    want = list(range(590, 600))
+    assert r.step([{"id": "a", "tokens": toks[:512], "want": []}]) is None
+    a = r.step([{"id": "a", "tokens": toks[512:], "want": [x - 512 for x in want]}], ["a"])
+    b = r.step([{"id": "b", "tokens": other, "want": want}], ["b"])
+    mostly(a, ref[want], dtype, "as it is")
+    mostly(b, ref2[want], dtype, "with token 3 changed")
+
+
+def test_greedy_generation_through_the_scheduler(gpu):
+    """``LLM.generate`` with temperature 0 gives the plain implementation's greedy tokens, for prompts of unequal
+    length in one call (32-bit, so that no rounding decides between neighbours)."""
+    from prelude_amd.llm import LLM
+    name = "p"
+    path, cfg, w = folder(name)
+    llm = LLM(path, dtype="float32", page_size=8, max_cache_tokens=512)
+    prompts = [plain_logits(name, 30, 9)[0], plain_logits(name, 31, 31)[0], plain_logits(name, 32, 2)[0]]
+    res = llm.generate(prompts, max_tokens=12, temperature=0.0)
+    for p, out in zip(prompts, res):
+        seq = list(p)
+        for _ in range(12):
+            seq.append(int(pf.forward(cfg, w, seq)[-1].argmax()))
+        assert out.token_ids == seq[len(p):], f"prompt of {len(p)}"
+
+
+def test_command_line_with_the_pools_sized_from_free_memory(gpu, capsys):
+    """``python -m prelude_amd`` on a Fazopel folder, nothing given but the model: the pools take what the device has
+    left after a measured step, and steps are replayed from graphs."""
+    from prelude_amd import cli
+    name = "q"
+    path, cfg, w = folder(name)
+    prompt = plain_logits(name, 40, 11)[0]
+    assert cli.main(["--model", path, "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "6", "--temperature", "0"]) == 0
+    rec = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert rec["finish_reason"] == "length" and len(rec["token_ids"]) == 6
+    ref = pf.forward(cfg, w, prompt)[-1]
+    top2 = torch.topk(ref, 2).values
+    if float(top2[0] - top2[1]) > 0.25 * float(ref.std()):
+        assert rec["token_ids"][0] == int(ref.argmax())
+    assert cli.main(["--model", path, "--random-weights", "--prompt-len", "5", "--max-tokens", "3", "--max-cache-tokens", "256"]) == 0
+    rec = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert len(rec["token_ids"]) == 3 and all(0 <= t < cfg["vocab"] for t in rec["token_ids"])
