@@ -85,6 +85,7 @@ _KERNEL_API = {
     "pa_moe_linear_mfma": (I, [P, I, P, P, P, P, P, I, I, I, I, I, I, I]),
     "pa_head_linear_mfma": (I, [P, P, P, P, I, I, I, I, c_long, c_long, c_long, c_long]),
     "pa_moe_combine": (I, [P, I, P, P, P, F, P, P, P, I, I, I]),
+    "pa_gemm_narrow": (I, [P, P, P, P, I, I, I, c_long, c_long]),
     "pa_moe_route": (I, [P, P, I, P, P, P, P, I, I, I, F, I]),
     "pa_qknorm_rope_kv_freq": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I]),
     "pa_attn_decode_sink": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, F, P, I, I]),

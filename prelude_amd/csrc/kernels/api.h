@@ -63,6 +63,9 @@ int pa_gemm_library(void* stream, const void* x, const void* w, void* c, int m, 
 int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, const void* w, const float* bias, void* c,
                   int m, int n, int k, long lda, long ldw, long ldc);
 
+// C[m, n] = X[m, k] W[n, k]^T for a weight of few rows (n <= 512), bfloat16 operands (k a multiple of 8), 32-bit sums
+// and result: what a router's scores want at any number of rows.
+int pa_gemm_narrow(void* stream, const void* x, const void* w, float* c, int m, int n, int k, long ldx, long ldc);
 // C[m, n] = X[m, k] W[n, k]^T for m <= 64 in bfloat16 (32-bit accumulation); out_dtype 0 = float32, 1 = bfloat16.
 // epilogue 0: (+ bias[n]); 1: C[m, n/2] = silu(gate) * up for a weight whose rows alternate gate_j, up_j.
 // tiled 1: w is the weight as pa_pack_tiles lays it out.

@@ -9,10 +9,11 @@
 // state slot state_slots[s]; a request's portions may be cut anywhere, the state carries over.
 //
 // pa_lightning_attn: the recurrence as it stands, on the vector ALU, for any sizes and both element types.  A
-// workgroup owns (64 value columns, head, sequence): four wavefronts split the rows of S between them (a quarter
-// each), each thread keeps its rows of one column in registers and walks the tokens in order, sixteen at a time
-// through LDS; the four partial dot products of a token are added in wavefront order.  The order of every sum
-// follows the token's place in its sequence alone, so a token's output is the same bits however its prompt was cut.
+// workgroup owns (64 or 128 value columns, head, sequence).  A lane keeps a quarter of the rows of S for one column
+// (or two, 64 apart) in registers: the 16-lane rows of a wavefront are the four quarters, its wavefront picks the 16
+// columns.  It walks the tokens in order, sixteen at a time through LDS; a token's four partial dot products are
+// added across the wavefront's rows, (0 + 1) + (2 + 3).  The order of every sum follows the token's place in its
+// sequence alone, so a token's output is the same bits however its prompt was cut.
 //
 // pa_lightning_attn_chunked: the same sums for long portions with the whole chip at work.  A portion is cut into
 // chunks of C tokens; with S_b the state before a chunk and i a token's place in it,
@@ -30,11 +31,21 @@
 namespace pa {
 
 constexpr int kLaTokens = 16;    // tokens staged at a time
-constexpr int kLaCols = 64;      // value columns a workgroup
-constexpr int kLaParts = 4;      // wavefronts, each with a quarter of the state's rows
+constexpr int kLaLanes = 64;     // value columns a workgroup, times NC
+constexpr int kLaThreads = 256;
 constexpr int kLaMaxChunk = 256;
 
 __device__ __forceinline__ float la_act(float x, int act) { return act == 1 ? x / (1.0f + expf(-x)) : x; }
+
+// The sum over the four 16-lane rows of a wavefront, (row 0 + row 1) + (row 2 + row 3), in every lane.
+__device__ __forceinline__ float la_sum_rows(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const unsigned w = __float_as_uint(v);
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
 
 enum LaMode : int { kLaWhole = 0, kLaLocal = 1, kLaApply = 2 };
 
@@ -43,23 +54,25 @@ enum LaMode : int { kLaWhole = 0, kLaLocal = 1, kLaApply = 2 };
 // below tokens / C + sequences.
 __device__ __forceinline__ size_t la_chunk_index(int row0, int chunk, int z, int j) { return (size_t)(row0 / chunk + z + j); }
 
-// R: rows of the state a thread keeps (dim <= 4 R, R a multiple of 4).
+// R: rows of the state a lane keeps (dim <= 4 R, R a multiple of 4); NC: columns a lane keeps (64 apart).
 // kLaWhole: grid (column tiles, heads, sequences); sequences longer than `max_len` tokens (> 0) are left alone.
 // kLaLocal / kLaApply: grid (column tiles, heads, listed sequences x max_chunks); sequences of at most one chunk and
 // chunks past a sequence's end leave at once.
-template <typename T, int R, int MODE>
-__global__ __launch_bounds__(kLaParts* kLaCols) void lightning_attn_kernel(
+template <typename T, int R, int NC, int MODE>
+__global__ __launch_bounds__(kLaThreads) void lightning_attn_kernel(
     const T* __restrict__ qkv, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_q,
     const int* __restrict__ seq_ids, float* __restrict__ out, float* __restrict__ work, int heads, int dim, int vdim, int act,
     int max_len, int chunk, int max_chunks) {
+  constexpr int kCols = kLaLanes * NC;
   __shared__ __align__(16) float qs[kLaTokens][4 * R];
-  __shared__ __align__(16) float ks[kLaTokens][4 * R];
-  __shared__ float vs[kLaTokens][kLaCols];
-  __shared__ float part[kLaParts][kLaTokens][kLaCols];
+  __shared__ __align__(16) float ks[MODE == kLaApply ? 1 : kLaTokens][4 * R];
+  __shared__ float vs[MODE == kLaApply ? 1 : kLaTokens][kCols];
   __shared__ float pw[MODE == kLaApply ? kLaMaxChunk : 1];
-  const int col = threadIdx.x % kLaCols, w = threadIdx.x / kLaCols;
-  const int c0 = blockIdx.x * kLaCols, h = blockIdx.y;
+  const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int dp = lane / 16;                      // which quarter of the rows
+  const int cl = 16 * w + lane % 16;             // column within a run of 64
+  const int c0 = blockIdx.x * kCols, h = blockIdx.y;
   int seq, z = 0, j = 0;
   if (MODE == kLaWhole) {
     seq = blockIdx.z;
@@ -73,28 +86,34 @@ __global__ __launch_bounds__(kLaParts* kLaCols) void lightning_attn_kernel(
   if (MODE == kLaWhole && max_len > 0 && row1 - row0 > max_len) return;
   float* sp;
   if (MODE == kLaWhole) {
-    sp = state + (((size_t)slot * heads + h) * dim) * vdim + c0 + col;
+    sp = state + (((size_t)slot * heads + h) * dim) * vdim;
   } else {
     if (row1 - row0 <= chunk || row0 + j * chunk >= row1) return;
-    sp = work + ((la_chunk_index(row0, chunk, z, j) * heads + h) * dim) * vdim + c0 + col;
+    sp = work + ((la_chunk_index(row0, chunk, z, j) * heads + h) * dim) * vdim;
     row0 += j * chunk;
     row1 = row1 < row0 + chunk ? row1 : row0 + chunk;
   }
-  const bool live = c0 + col < vdim;
   const float a = decay[h];
   if (MODE == kLaApply) {
-    for (int i = threadIdx.x; i < chunk; i += kLaParts * kLaCols) pw[i] = powf(a, (float)(i + 1));
+    for (int i = threadIdx.x; i < chunk; i += kLaThreads) pw[i] = powf(a, (float)(i + 1));
   }
-  float S[R];
+  int col[NC];
+  bool live[NC];
+  float S[NC][R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int d = w * R + r;
-    S[r] = (MODE != kLaLocal && live && d < dim) ? sp[(size_t)d * vdim] : 0.f;
+  for (int c = 0; c < NC; ++c) {
+    col[c] = c0 + kLaLanes * c + cl;
+    live[c] = col[c] < vdim;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int d = dp * R + r;
+      S[c][r] = (MODE != kLaLocal && live[c] && d < dim) ? sp[(size_t)d * vdim + col[c]] : 0.f;
+    }
   }
   for (int t0 = row0; t0 < row1; t0 += kLaTokens) {
     const int n = row1 - t0 < kLaTokens ? row1 - t0 : kLaTokens;
     __syncthreads();   // the block before has been read
-    for (int i = threadIdx.x; i < n * 4 * R; i += kLaParts * kLaCols) {
+    for (int i = threadIdx.x; i < n * 4 * R; i += kLaThreads) {
       const int t = i / (4 * R), d = i % (4 * R);
       float qv = 0.f, kv = 0.f;   // rows past dim are zeros: they leave the sums alone
       if (d < dim) {
@@ -106,52 +125,53 @@ __global__ __launch_bounds__(kLaParts* kLaCols) void lightning_attn_kernel(
       if (MODE != kLaApply) ks[t][d] = kv;
     }
     if (MODE != kLaApply) {
-      for (int i = threadIdx.x; i < n * kLaCols; i += kLaParts * kLaCols) {
-        const int t = i / kLaCols, c = i % kLaCols;
+      for (int i = threadIdx.x; i < n * kCols; i += kLaThreads) {
+        const int t = i / kCols, c = i % kCols;
         vs[t][c] = c0 + c < vdim ? la_act(to_f32(qkv[(size_t)(t0 + t) * ld + v_off + (size_t)h * vdim + c0 + c]), act) : 0.f;
       }
     }
     __syncthreads();
     for (int t = 0; t < n; ++t) {
-      float acc = 0.f;
-      if (MODE == kLaApply) {
+      float acc[NC];
+      float v[NC];
 #pragma unroll
-        for (int r = 0; r < R; r += 4) {
-          const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[t][w * R + r]);
+      for (int c = 0; c < NC; ++c) {
+        acc[c] = 0.f;
+        v[c] = MODE == kLaApply ? 0.f : vs[t][kLaLanes * c + cl];
+      }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc = fmaf(S[r + e], q4[e], acc);
-        }
-      } else {
-        const float v = vs[t][col];
+      for (int r = 0; r < R; r += 4) {
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[t][dp * R + r]);
+        f32x4 k4 = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (MODE != kLaApply) k4 = *reinterpret_cast<const f32x4*>(&ks[t][dp * R + r]);
 #pragma unroll
-        for (int r = 0; r < R; r += 4) {
-          const f32x4 k4 = *reinterpret_cast<const f32x4*>(&ks[t][w * R + r]);
-          const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[t][w * R + r]);
+        for (int e = 0; e < 4; ++e) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            S[r + e] = fmaf(a, S[r + e], k4[e] * v);
-            acc = fmaf(S[r + e], q4[e], acc);
+          for (int c = 0; c < NC; ++c) {
+            if (MODE != kLaApply) S[c][r + e] = fmaf(a, S[c][r + e], k4[e] * v[c]);
+            acc[c] = fmaf(S[c][r + e], q4[e], acc[c]);
           }
         }
       }
-      part[w][t][col] = acc;
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < n * kLaCols; i += kLaParts * kLaCols) {
-      const int t = i / kLaCols, c = i % kLaCols;
-      if (c0 + c < vdim) {
-        const float sum = ((part[0][t][c] + part[1][t][c]) + part[2][t][c]) + part[3][t][c];
-        float* o = out + ((size_t)(t0 + t) * heads + h) * vdim + c0 + c;
-        if (MODE == kLaApply) *o += pw[t0 + t - row0] * sum;
-        else *o = sum;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const float sum = la_sum_rows(acc[c]);
+        if (dp == 0 && live[c]) {
+          float* o = out + ((size_t)(t0 + t) * heads + h) * vdim + col[c];
+          if (MODE == kLaApply) *o += pw[t0 + t - row0] * sum;
+          else *o = sum;
+        }
       }
     }
   }
-  if (MODE != kLaApply && live) {
+  if (MODE != kLaApply) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int d = w * R + r;
-      if (d < dim) sp[(size_t)d * vdim] = S[r];
+    for (int c = 0; c < NC; ++c) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int d = dp * R + r;
+        if (live[c] && d < dim) sp[(size_t)d * vdim + col[c]] = S[c][r];
+      }
     }
   }
 }
@@ -185,17 +205,21 @@ __global__ __launch_bounds__(256) void lightning_scan_kernel(const float* __rest
 }
 
 template <typename T, int MODE>
-static void launch_lightning(hipStream_t st, dim3 grid, const T* qkv, long ld, int q_off, int k_off, int v_off,
+static void launch_lightning(hipStream_t st, int zdim, const T* qkv, long ld, int q_off, int k_off, int v_off,
                              const float* decay, float* state, const int* state_slots, const int* cu_q, const int* seq_ids,
                              float* out, float* work, int heads, int dim, int vdim, int act, int max_len, int chunk,
                              int max_chunks) {
-#define PA_LA(R)                                                                                                          \
-  hipLaunchKernelGGL((lightning_attn_kernel<T, R, MODE>), grid, dim3(kLaParts* kLaCols), 0, st, qkv, ld, q_off, k_off,     \
-                     v_off, decay, state, state_slots, cu_q, seq_ids, out, work, heads, dim, vdim, act, max_len, chunk, max_chunks)
-  if (dim <= 32) PA_LA(8);
-  else if (dim <= 64) PA_LA(16);
-  else if (dim <= 128) PA_LA(32);
-  else PA_LA(64);
+  // two columns a lane where the state is wide enough and its rows leave the registers for them
+  const bool two = vdim > kLaLanes && dim <= 128;
+  const int cols = two ? 2 * kLaLanes : kLaLanes;
+  dim3 grid((vdim + cols - 1) / cols, heads, zdim);
+#define PA_LA(R, NC)                                                                                                       \
+  hipLaunchKernelGGL((lightning_attn_kernel<T, R, NC, MODE>), grid, dim3(kLaThreads), 0, st, qkv, ld, q_off, k_off, v_off, \
+                     decay, state, state_slots, cu_q, seq_ids, out, work, heads, dim, vdim, act, max_len, chunk, max_chunks)
+  if (dim <= 32) { if (two) PA_LA(8, 2); else PA_LA(8, 1); }
+  else if (dim <= 64) { if (two) PA_LA(16, 2); else PA_LA(16, 1); }
+  else if (dim <= 128) { if (two) PA_LA(32, 2); else PA_LA(32, 1); }
+  else PA_LA(64, 1);
 #undef PA_LA
 }
 
@@ -222,12 +246,11 @@ extern "C" int pa_lightning_attn(void* stream, int dtype, const void* qkv, long 
   if (int rc = lightning_check("lightning_attn", nseq, tokens, heads, dim, vdim, ld, q_off, k_off, v_off, act)) return rc;
   PA_REQUIRE(nseq <= 65535, "lightning_attn: %d sequences exceed the grid", nseq);
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((vdim + kLaCols - 1) / kLaCols, heads, nseq);
   if (dtype == kF32)
-    launch_lightning<float, kLaWhole>(st, grid, (const float*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
+    launch_lightning<float, kLaWhole>(st, nseq, (const float*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
                                       nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1);
   else if (dtype == kBF16)
-    launch_lightning<bf16, kLaWhole>(st, grid, (const bf16*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
+    launch_lightning<bf16, kLaWhole>(st, nseq, (const bf16*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
                                      nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1);
   else
     return pa::fail("lightning_attn: unknown element type code %d", dtype);
@@ -253,11 +276,10 @@ extern "C" int pa_lightning_attn_chunked(void* stream, int dtype, const void* qk
   const int max_chunks = (max_len + chunk - 1) / chunk;
   PA_REQUIRE((long)nlisted * max_chunks <= 65535, "lightning_attn_chunked: %d sequences x %d chunks exceed the grid", nlisted, max_chunks);
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((vdim + kLaCols - 1) / kLaCols, heads, nlisted * max_chunks);
   const int per_head = dim * vdim;
   dim3 scan_grid((per_head + 255) / 256, heads, nlisted);
 #define PA_LA_PASS(T, MODE)                                                                                               \
-  launch_lightning<T, MODE>(st, grid, (const T*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q, seq_ids, out, \
+  launch_lightning<T, MODE>(st, nlisted * max_chunks, (const T*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q, seq_ids, out, \
                             work, heads, dim, vdim, act, 0, chunk, max_chunks)
 #define PA_LA_SCAN()                                                                                                      \
   hipLaunchKernelGGL(lightning_scan_kernel, scan_grid, dim3(256), 0, st, decay, state, state_slots, cu_q, seq_ids, work,   \

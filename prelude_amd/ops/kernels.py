@@ -1163,7 +1163,7 @@ def gated_rmsnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps
 LIGHTNING_ACTIVATIONS = {None: 0, "none": 0, "silu": 1}
 
 
-LIGHTNING_CHUNK = 128      # tokens a chunk of the chunked form; portions of more tokens go to it (bfloat16 engine)
+LIGHTNING_CHUNK = 64       # tokens a chunk of the chunked form; portions of more tokens go to it (bfloat16 engine)
 
 
 def lightning_attention(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, state: torch.Tensor,
@@ -1358,6 +1358,29 @@ def moe_choices_by_table(token_ids: torch.Tensor, table: torch.Tensor, experts: 
     check(kernels().pa_moe_choices_by_table(_stream(), _ptr(token_ids), _ptr(table), _ptr(choice), t, top, table.shape[0],
                                             int(experts)))
     return choice
+
+
+NARROW_MAX_COLUMNS = 512
+NARROW_FEW_ROWS = 16     # up to here the weight-streaming product (32-bit result from its own sums) is the faster one
+
+
+def linear_narrow_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x W^T for a weight of few rows with a 32-bit result from 32-bit sums, whatever the number of rows of x: a
+    router's scores (the library's product would round them to bfloat16).  float32: the plain product.  bfloat16:
+    few rows the weight-streaming kernel, more the matrix-core kernel for narrow outputs; sizes neither takes
+    (rows of no whole 16-byte pieces, more than ``NARROW_MAX_COLUMNS`` columns) go to the plain product too."""
+    _dev(x, w)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.dtype != w.dtype:
+        raise NativeError(f"linear_narrow_f32: x {tuple(x.shape)} {x.dtype} / w {tuple(w.shape)} {w.dtype}")
+    m, k = x.shape
+    n = w.shape[0]
+    if x.dtype != torch.bfloat16 or k % 8 or n > NARROW_MAX_COLUMNS:
+        return gemm_plain(x, w, None, torch.float32)
+    if m <= NARROW_FEW_ROWS:
+        return gemm_skinny(x, w, None, torch.float32)
+    out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    check(kernels().pa_gemm_narrow(_stream(), _ptr(x), _ptr(w), _ptr(out), m, n, k, k, n))
+    return out
 
 
 def moe_route(logits: torch.Tensor, experts: int, top: int, scale: float, correction: Optional[torch.Tensor] = None,

@@ -130,9 +130,8 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, step=None):
         n = self.num_experts
-        # the router's sums are 32-bit in a fixed order whatever the number of rows (the operands are of the engine's
-        # type): a product of few columns, for which the plain kernel is the right one
-        logits = K.gemm_plain(x, self.router, None, torch.float32)
+        # the router's sums and scores are 32-bit (the operands are of the engine's type): a product of few columns
+        logits = K.linear_narrow_f32(x, self.router)
         choice, weights, gate = K.moe_route(logits, n, self.top, self.route_scale, self.correction,
                                             gate_col=n if self.shared_size else -1)
         eo = K.moe_order(choice, n, self.top)
