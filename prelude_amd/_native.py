@@ -82,7 +82,7 @@ _KERNEL_API = {
     "pa_moe_choices_by_table": (I, [P, P, P, P, I, I, I, I]),
     "pa_moe_order": (I, [P, P, I, I, P, P, P, P]),
     "pa_moe_linear": (I, [P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I]),
-    "pa_moe_linear_mfma": (I, [P, I, P, P, P, P, P, I, I, I, I, I, I, I]),
+    "pa_moe_linear_mfma": (I, [P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, F]),
     "pa_head_linear_mfma": (I, [P, P, P, P, I, I, I, I, c_long, c_long, c_long, c_long]),
     "pa_moe_combine": (I, [P, I, P, P, P, F, P, P, P, I, I, I]),
     "pa_gemm_narrow": (I, [P, P, P, P, I, I, I, c_long, c_long]),

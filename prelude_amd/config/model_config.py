@@ -334,7 +334,7 @@ class FazopelLayerConfig:
     type: str                   # "lightning" | "attention"
     mixer: object               # LightningMixerConfig | SinkAttentionConfig
     mlp: Optional[FazopelMlpConfig]
-    weights_of: Optional[int]   # the layer whose tensors this one uses (its own cache or state); None: its own
+    weights_of: Optional[int]   # the layer whose tensors this one uses (its own cache or state), itself a layer with tensors; None: its own
 
 
 @dataclasses.dataclass(frozen=True)
@@ -358,9 +358,12 @@ class FazopelConfig:
         a = cls.ARCH
         heads = _positive(m, "heads", int, a, mw)
         dim = _positive(m, "dim", int, a, mw)
-        vdim = _positive(m, "vdim", int, a, mw)
+        # the values of the attention are its keys, so their size is the keys' and may go unsaid
+        vdim = _positive(m, "vdim", int, a, mw) if (kind == "lightning" or m.get("vdim") is not None) else dim
         if kind == "lightning":
             decay = m.get("decay")
+            if isinstance(decay, (int, float)) and not isinstance(decay, bool):
+                decay = [decay] * heads          # one number for all heads
             if not isinstance(decay, list) or len(decay) != heads or \
                     not all(isinstance(x, (int, float)) and not isinstance(x, bool) and 0.0 <= x <= 1.0 for x in decay):
                 raise ConfigError(f"failed to parse {a} config: `{mw}decay` must list one number in [0, 1] for each of "
@@ -432,14 +435,15 @@ class FazopelConfig:
                     raise ConfigError(f"failed to parse {a} config: `{w}weights_of` ({src}) names no other layer")
             layers.append(layer)
         for i, layer in enumerate(layers):
-            if layer.weights_of is not None:
-                j = layer.weights_of
-                if layers[j].weights_of is not None:
-                    raise ConfigError(f"failed to parse {a} config: `layers[{i}].weights_of` names layer {j}, which has no "
-                                      f"tensors of its own")
-                if dataclasses.replace(layers[j], weights_of=None) != dataclasses.replace(layer, weights_of=None):
-                    raise ConfigError(f"failed to parse {a} config: `layers[{i}]` uses the tensors of layer {j} but "
-                                      f"differs from it")
+            # a layer may name one that itself names another: the tensors are those of the end of the chain
+            j, seen = layer.weights_of, {i}
+            while j is not None and layers[j].weights_of is not None:
+                if j in seen:
+                    raise ConfigError(f"failed to parse {a} config: `layers[{i}].weights_of` leads in a circle")
+                seen.add(j)
+                j = layers[j].weights_of
+            if j is not None and j != layer.weights_of:
+                layers[i] = dataclasses.replace(layer, weights_of=j)
         norm = _obj(raw, "norm", a)
         return cls(vocab=_positive(raw, "vocab", int, a, ""), width=_positive(raw, "width", int, a, ""),
                    norm_eps=_positive(norm, "eps", float, a, "norm."), layers=tuple(layers))

@@ -63,7 +63,7 @@ int pa_gemm_library(void* stream, const void* x, const void* w, void* c, int m, 
 int pa_gemm_plain(void* stream, int in_dtype, int out_dtype, const void* a, const void* w, const float* bias, void* c,
                   int m, int n, int k, long lda, long ldw, long ldc);
 
-// C[m, n] = X[m, k] W[n, k]^T for a weight of few rows (n <= 512), bfloat16 operands (k a multiple of 8), 32-bit sums
+// C[m, n] = X[m, k] W[n, k]^T for a weight of few rows (n <= 256), bfloat16 operands (k a multiple of 8), 32-bit sums
 // and result: what a router's scores want at any number of rows.
 int pa_gemm_narrow(void* stream, const void* x, const void* w, float* c, int m, int n, int k, long ldx, long ldc);
 // C[m, n] = X[m, k] W[n, k]^T for m <= 64 in bfloat16 (32-bit accumulation); out_dtype 0 = float32, 1 = bfloat16.
@@ -270,8 +270,10 @@ int pa_moe_route(void* stream, const float* logits, int ld, const float* correct
                  float* gate_out, int tokens, int experts, int top, float scale, int gate_col);
 // The same two products on the matrix cores (grouped_mfma.hip; bfloat16 operands, K a multiple of 8): the weight as
 // stored, [group, N, K].
+// act 2 (here only): the weight's rows alternate gate_j, up_j and y [entries, N / 2] receives the clamped gated pair
+// g * sigmoid(alpha g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit).
 int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, const void* w, void* y, const int* offsets, const int* order,
-                       int entries, int experts, int top, int K, int N, int from_tokens, int act);
+                       int entries, int experts, int top, int K, int N, int from_tokens, int act, float limit, float alpha);
 int pa_head_linear_mfma(void* stream, const void* x, const void* w, void* y, int tokens, int heads, int K, int N, long xs_t,
                         long xs_h, long ys_t, long ys_h);
 

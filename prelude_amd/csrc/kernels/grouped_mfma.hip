@@ -20,7 +20,7 @@ constexpr int kGmRows = 64;
 // xrow(m) / yrow(m): element offsets of row m's input and output, < 0 for a row that does not exist.
 template <typename TY, int NT, typename RowX, typename RowY>
 __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const bf16* __restrict__ w, TY* __restrict__ y,
-                                             int K, int N, int n_rows, int n0, int act, RowX xrow, RowY yrow) {
+                                             int K, int N, int n_rows, int n0, int act, float limit, float alpha, RowX xrow, RowY yrow) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int row_tiles = (n_rows + 15) / 16;
@@ -98,6 +98,10 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
         const int n = nb + 16 * j + 4 * g + i;
         if (n < N) {
           float v = acc[j][mt][i];
+          if (act == 2) {   // a lane's four outputs are two (gate, up) pairs: one output a pair, rows of N / 2
+            if ((i & 1) == 0) y[yo + n / 2] = from_f32<TY>(clamped_gate(v, acc[j][mt][i | 1], limit, alpha));
+            continue;
+          }
           if (act == 1) {
             v = fmaxf(v, 0.f);
             v = v * v;
@@ -151,7 +155,8 @@ template <typename TY, int NT>
 __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                              TY* __restrict__ y, const int* __restrict__ offsets,
                                                              const int* __restrict__ order, int entries, int experts,
-                                                             int top, int K, int N, int col_chunks, int from_tokens, int act) {
+                                                             int top, int K, int N, int col_chunks, int from_tokens, int act,
+                                                             float limit, float alpha) {
   // The launch is a line of workgroups that the hardware deals out to the eight XCDs in turn (each with an L2 of
   // its own); work item w = (chunk of outputs, tile of positions), tiles fastest, and every XCD is given one stretch
   // of the items: the tiles of one expert against one chunk of its weight then run on one XCD one after the other,
@@ -164,9 +169,9 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __rest
   int e = 0, p0 = 0, p1 = 0;
   const int col_chunk = item / tiles_max;
   if (!find_tile(offsets, experts, kGmRows, item % tiles_max, e, p0, p1)) return;
-  grouped_tile<TY, NT>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, col_chunk * 64 * NT, act,
+  grouped_tile<TY, NT>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, col_chunk * 64 * NT, act, limit, alpha,
                    [&](int m) { return (long)(from_tokens ? order[p0 + m] / top : p0 + m) * K; },
-                   [&](int m) { return (long)(p0 + m) * N; });
+                   [&](int m) { return (long)(p0 + m) * (act == 2 ? N / 2 : N); });
 }
 
 // The experts' product for many rows: a workgroup owns 128 positions of one expert and 128 outputs.  What limits
@@ -182,7 +187,7 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_big_kernel(const bf16* __
                                                                  TY* __restrict__ y, const int* __restrict__ offsets,
                                                                  const int* __restrict__ order, int entries, int experts,
                                                                  int top, int K, int N, int col_chunks, int from_tokens,
-                                                                 int act) {
+                                                                 int act, float limit, float alpha) {
   __shared__ __attribute__((aligned(16))) bf16 xs[2][kGbRows * kGbStride];
   const int tiles_max = (entries + kGbRows - 1) / kGbRows + experts;
   const int total = tiles_max * col_chunks;
@@ -281,7 +286,7 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_big_kernel(const bf16* __
 #pragma unroll
   for (int mt = 0; mt < 8; ++mt) {
     if (mt * 16 + r >= n_rows) continue;
-    TY* yr = y + (size_t)(p0 + mt * 16 + r) * N;
+    TY* yr = y + (size_t)(p0 + mt * 16 + r) * (act == 2 ? N / 2 : N);
 #pragma unroll
     for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -289,6 +294,10 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_big_kernel(const bf16* __
         const int n = nb + 16 * j + 4 * g + i;
         if (n < N) {
           float v = acc[j][mt][i];
+          if (act == 2) {
+            if ((i & 1) == 0) yr[n / 2] = from_f32<TY>(clamped_gate(v, acc[j][mt][i | 1], limit, alpha));
+            continue;
+          }
           if (act == 1) {
             v = fmaxf(v, 0.f);
             v = v * v;
@@ -306,7 +315,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __res
                                                               long xs_h, long ys_t, long ys_h) {
   const int t0 = blockIdx.x * kGmRows, h = blockIdx.y;
   const int n_rows = tokens - t0 < kGmRows ? tokens - t0 : kGmRows;
-  grouped_tile<bf16, NT>(x, w + (size_t)h * N * K, y, K, N, n_rows, blockIdx.z * 64 * NT, 0,
+  grouped_tile<bf16, NT>(x, w + (size_t)h * N * K, y, K, N, n_rows, blockIdx.z * 64 * NT, 0, 0.f, 0.f,
                      [&](int m) { return (long)(t0 + m) * xs_t + (long)h * xs_h; },
                      [&](int m) { return (long)(t0 + m) * ys_t + (long)h * ys_h; });
 }
@@ -318,11 +327,13 @@ using namespace pa;
 // x [rows, K] bfloat16 (a row per token when from_tokens, else per position), w [experts, N, K] bfloat16,
 // y [entries, N] of y_dtype; K a multiple of 8.
 extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, const void* w, void* y, const int* offsets,
-                                  const int* order, int entries, int experts, int top, int K, int N, int from_tokens, int act) {
+                                  const int* order, int entries, int experts, int top, int K, int N, int from_tokens, int act,
+                                  float limit, float alpha) {
   if (entries == 0) return 0;
   PA_REQUIRE(entries > 0 && experts > 0 && top > 0 && K > 0 && N > 0 && K % 8 == 0, "moe_linear_mfma: bad sizes entries=%d experts=%d k=%d n=%d",
              entries, experts, K, N);
-  PA_REQUIRE(act == 0 || act == 1, "moe_linear_mfma: unknown activation code %d", act);
+  PA_REQUIRE(act == 0 || act == 1 || act == 2, "moe_linear_mfma: unknown activation code %d", act);
+  PA_REQUIRE(act != 2 || (N % 2 == 0 && limit > 0.f), "moe_linear_mfma: gated pairs need an even number of outputs and a clamp > 0");
   const bool few = entries <= 4 * kGmRows;
   const int cols = 128;
   const int col_chunks = (N + cols - 1) / cols;
@@ -334,10 +345,10 @@ extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, cons
     dim3 grid((unsigned)(((items + 7) / 8) * 8));
     if (y_dtype == kBF16)
       hipLaunchKernelGGL(moe_linear_mfma_big_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (bf16*)y, offsets,
-                         order, entries, experts, top, K, N, col_chunks, from_tokens, act);
+                         order, entries, experts, top, K, N, col_chunks, from_tokens, act, limit, alpha);
     else if (y_dtype == kF32)
       hipLaunchKernelGGL(moe_linear_mfma_big_kernel<float>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (float*)y, offsets,
-                         order, entries, experts, top, K, N, col_chunks, from_tokens, act);
+                         order, entries, experts, top, K, N, col_chunks, from_tokens, act, limit, alpha);
     else
       return pa::fail("moe_linear_mfma: unknown output type code %d", y_dtype);
     return check_launch("moe_linear_mfma");
@@ -347,7 +358,7 @@ extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, cons
   dim3 grid((unsigned)(((items + 7) / 8) * 8));
 #define PA_GM(TY, NT)                                                                                                       \
   hipLaunchKernelGGL((moe_linear_mfma_kernel<TY, NT>), grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w, (TY*)y, offsets, \
-                     order, entries, experts, top, K, N, col_chunks, from_tokens, act)
+                     order, entries, experts, top, K, N, col_chunks, from_tokens, act, limit, alpha)
   if (y_dtype == kBF16) {
     PA_GM(bf16, 2);
   } else if (y_dtype == kF32) {

@@ -59,14 +59,17 @@ __device__ __forceinline__ size_t la_chunk_index(int row0, int chunk, int z, int
 // kLaLocal / kLaApply: grid (column tiles, heads, listed sequences x max_chunks); sequences of at most one chunk and
 // chunks past a sequence's end leave at once.
 template <typename T, int R, int NC, int MODE>
-__global__ __launch_bounds__(kLaThreads) void lightning_attn_kernel(
+__global__ __launch_bounds__(kLaThreads, 2) void lightning_attn_kernel(
     const T* __restrict__ qkv, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_q,
     const int* __restrict__ seq_ids, float* __restrict__ out, float* __restrict__ work, int heads, int dim, int vdim, int act,
     int max_len, int chunk, int max_chunks) {
   constexpr int kCols = kLaLanes * NC;
-  __shared__ __align__(16) float qs[kLaTokens][4 * R];
-  __shared__ __align__(16) float ks[MODE == kLaApply ? 1 : kLaTokens][4 * R];
+  // a quarter's rows lie R + 4 floats apart: the four 16-byte reads of a wavefront (one a quarter) then fall into
+  // different banks (R is a multiple of 8, so R floats apart they would all fall into the same four)
+  constexpr int kQuarter = R + 4;
+  __shared__ __align__(16) float qs[kLaTokens][4 * kQuarter];
+  __shared__ __align__(16) float ks[MODE == kLaApply ? 1 : kLaTokens][4 * kQuarter];
   __shared__ float vs[MODE == kLaApply ? 1 : kLaTokens][kCols];
   __shared__ float pw[MODE == kLaApply ? kLaMaxChunk : 1];
   const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -110,57 +113,105 @@ __global__ __launch_bounds__(kLaThreads) void lightning_attn_kernel(
       S[c][r] = (MODE != kLaLocal && live[c] && d < dim) ? sp[(size_t)d * vdim + col[c]] : 0.f;
     }
   }
+  // A block of sixteen tokens on its way from memory: element e of the block is token e / kPerToken's query row d,
+  // key row d or value column, by its place inside the token.  All of a thread's loads are asked for together, a
+  // block ahead of their use, so the walk over a block's tokens hides them.
+  constexpr int kPerToken = (MODE == kLaApply ? 4 * R : 8 * R + kCols);
+  constexpr int kRaw = (kLaTokens * kPerToken + kLaThreads - 1) / kLaThreads;
+  T raw[kRaw];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < kRaw; ++i) {
+      const int e = threadIdx.x + kLaThreads * i;
+      const int t = e / kPerToken, x = e % kPerToken;
+      T v = from_f32<T>(0.f);   // rows past dim, columns past vdim and tokens past the end are zeros: they leave the sums alone
+      if (t0 + t < row1 && t < kLaTokens) {
+        const T* src = qkv + (size_t)(t0 + t) * ld;
+        if (x < 4 * R) {
+          if (x < dim) v = src[q_off + (size_t)h * dim + x];
+        } else if (x < 8 * R) {
+          if (x - 4 * R < dim) v = src[k_off + (size_t)h * dim + x - 4 * R];
+        } else if (c0 + x - 8 * R < vdim) {
+          v = src[v_off + (size_t)h * vdim + c0 + x - 8 * R];
+        }
+      }
+      raw[i] = v;
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < kRaw; ++i) {
+      const int e = threadIdx.x + kLaThreads * i;
+      const int t = e / kPerToken, x = e % kPerToken;
+      if (t >= kLaTokens) continue;
+      const float v = la_act(to_f32(raw[i]), act);
+      if (x < 4 * R) {
+        qs[t][(x / R) * kQuarter + x % R] = v;
+      } else if (MODE != kLaApply) {
+        if (x < 8 * R) ks[t][((x - 4 * R) / R) * kQuarter + (x - 4 * R) % R] = v;
+        else vs[t][x - 8 * R] = v;
+      }
+    }
+  };
+  fetch(row0);
   for (int t0 = row0; t0 < row1; t0 += kLaTokens) {
     const int n = row1 - t0 < kLaTokens ? row1 - t0 : kLaTokens;
     __syncthreads();   // the block before has been read
-    for (int i = threadIdx.x; i < n * 4 * R; i += kLaThreads) {
-      const int t = i / (4 * R), d = i % (4 * R);
-      float qv = 0.f, kv = 0.f;   // rows past dim are zeros: they leave the sums alone
-      if (d < dim) {
-        const T* src = qkv + (size_t)(t0 + t) * ld + (size_t)h * dim + d;
-        qv = la_act(to_f32(src[q_off]), act);
-        if (MODE != kLaApply) kv = la_act(to_f32(src[k_off]), act);
-      }
-      qs[t][d] = qv;
-      if (MODE != kLaApply) ks[t][d] = kv;
-    }
-    if (MODE != kLaApply) {
-      for (int i = threadIdx.x; i < n * kCols; i += kLaThreads) {
-        const int t = i / kCols, c = i % kCols;
-        vs[t][c] = c0 + c < vdim ? la_act(to_f32(qkv[(size_t)(t0 + t) * ld + v_off + (size_t)h * vdim + c0 + c]), act) : 0.f;
-      }
-    }
+    stage();
     __syncthreads();
-    for (int t = 0; t < n; ++t) {
-      float acc[NC];
-      float v[NC];
+    if (t0 + kLaTokens < row1) fetch(t0 + kLaTokens);
+    // The block's tokens in groups whose results leave together.  The third pass adds to what the stream holds: it
+    // asks for a whole block's places before the walk (its state is fixed, so it has the registers); the passes
+    // that carry the state along take four tokens at a time, which keeps two wavefronts on a SIMD.
+    constexpr int kGroup = MODE == kLaApply ? kLaTokens : 4;
+#pragma unroll 1
+    for (int tb = 0; tb < n; tb += kGroup) {
+      float res[kGroup][NC];
+      if (MODE == kLaApply) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        acc[c] = 0.f;
-        v[c] = MODE == kLaApply ? 0.f : vs[t][kLaLanes * c + cl];
+        for (int u = 0; u < kGroup; ++u)
+#pragma unroll
+          for (int c = 0; c < NC; ++c)
+            res[u][c] = (dp == 0 && live[c] && tb + u < n) ? out[((size_t)(t0 + tb + u) * heads + h) * vdim + col[c]] : 0.f;
       }
 #pragma unroll
-      for (int r = 0; r < R; r += 4) {
-        const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[t][dp * R + r]);
-        f32x4 k4 = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (MODE != kLaApply) k4 = *reinterpret_cast<const f32x4*>(&ks[t][dp * R + r]);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
+      for (int u = 0; u < kGroup; ++u) {
+        const int t = tb + u;
+        if (t < n) {
+          float acc[NC];
+          float v[NC];
 #pragma unroll
           for (int c = 0; c < NC; ++c) {
-            if (MODE != kLaApply) S[c][r + e] = fmaf(a, S[c][r + e], k4[e] * v[c]);
-            acc[c] = fmaf(S[c][r + e], q4[e], acc[c]);
+            acc[c] = 0.f;
+            v[c] = MODE == kLaApply ? 0.f : vs[t][kLaLanes * c + cl];
+          }
+#pragma unroll
+          for (int r = 0; r < R; r += 4) {
+            const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[t][dp * kQuarter + r]);
+            f32x4 k4 = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (MODE != kLaApply) k4 = *reinterpret_cast<const f32x4*>(&ks[t][dp * kQuarter + r]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+#pragma unroll
+              for (int c = 0; c < NC; ++c) {
+                if (MODE != kLaApply) S[c][r + e] = fmaf(a, S[c][r + e], k4[e] * v[c]);
+                acc[c] = fmaf(S[c][r + e], q4[e], acc[c]);
+              }
+            }
+          }
+#pragma unroll
+          for (int c = 0; c < NC; ++c) {
+            const float sum = la_sum_rows(acc[c]);
+            res[u][c] = MODE == kLaApply ? res[u][c] + pw[t0 + t - row0] * sum : sum;
           }
         }
       }
+      if (dp == 0) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const float sum = la_sum_rows(acc[c]);
-        if (dp == 0 && live[c]) {
-          float* o = out + ((size_t)(t0 + t) * heads + h) * vdim + col[c];
-          if (MODE == kLaApply) *o += pw[t0 + t - row0] * sum;
-          else *o = sum;
-        }
+        for (int u = 0; u < kGroup; ++u)
+#pragma unroll
+          for (int c = 0; c < NC; ++c)
+            if (tb + u < n && live[c]) out[((size_t)(t0 + tb + u) * heads + h) * vdim + col[c]] = res[u][c];
       }
     }
   }

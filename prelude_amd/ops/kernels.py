@@ -1360,7 +1360,7 @@ def moe_choices_by_table(token_ids: torch.Tensor, table: torch.Tensor, experts: 
     return choice
 
 
-NARROW_MAX_COLUMNS = 512
+NARROW_MAX_COLUMNS = 256
 NARROW_FEW_ROWS = 16     # up to here the weight-streaming product (32-bit result from its own sums) is the faster one
 
 
@@ -1415,23 +1415,33 @@ def moe_order(choice: torch.Tensor, experts: int, top: int) -> ExpertOrder:
 
 
 def moe_linear(x: torch.Tensor, w: GroupedWeight, eo: ExpertOrder, from_tokens: bool, relu_squared_epilogue: bool = False,
-               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+               out_dtype: Optional[torch.dtype] = None, clamped_gate_epilogue: Optional[tuple] = None) -> torch.Tensor:
     """y[p] = act(W[expert of p] x[row of p]) over the ordered positions p; ``w`` [experts, n, k];
-    ``from_tokens``: x holds a row per token (position p reads its token's), else a row per position."""
+    ``from_tokens``: x holds a row per token (position p reads its token's), else a row per position.
+    ``clamped_gate_epilogue`` = (limit, alpha): the weights' rows alternate gate_j, up_j and the result is the
+    clamped gated pair of ``clamped_gate``, [entries, n / 2] (in the matrix-core product's epilogue; a kernel of
+    its own behind the other product)."""
     wt = w.nk if w.nk is not None else w.kn
     _dev(x, wt)
     k, n = w.k, w.n
     rows = eo.entries // eo.top if from_tokens else eo.entries
     if x.dim() != 2 or tuple(x.shape) != (rows, k) or w.groups != eo.experts or x.dtype != w.dtype:
         raise NativeError(f"moe_linear: x {tuple(x.shape)} {x.dtype} / w [{w.groups}, {n}, {k}] {w.dtype} for {eo.entries} entries")
+    if clamped_gate_epilogue is not None and (relu_squared_epilogue or n % 2):
+        raise NativeError(f"moe_linear: gated pairs over {n} outputs, or two activations at once")
     out_dtype = out_dtype or x.dtype
-    y = torch.empty((eo.entries, n), dtype=out_dtype, device=x.device)
+    fused = clamped_gate_epilogue is not None and w.nk is not None
+    y = torch.empty((eo.entries, n // 2 if fused else n), dtype=out_dtype, device=x.device)
+    act = 2 if fused else (1 if relu_squared_epilogue else 0)
     args = (_ptr(x), _ptr(wt), _ptr(y), _ptr(eo.offsets), _ptr(eo.order), eo.entries, eo.experts, eo.top, k, n,
-            1 if from_tokens else 0, 1 if relu_squared_epilogue else 0)
+            1 if from_tokens else 0, act)
     if w.nk is not None:
-        check(kernels().pa_moe_linear_mfma(_stream(), _CODES[out_dtype], *args))
-    else:
-        check(kernels().pa_moe_linear(_stream(), _code(x), _code(wt), _CODES[out_dtype], *args))
+        limit, alpha = clamped_gate_epilogue if fused else (0.0, 0.0)
+        check(kernels().pa_moe_linear_mfma(_stream(), _CODES[out_dtype], *args, float(limit), float(alpha)))
+        return y
+    check(kernels().pa_moe_linear(_stream(), _code(x), _code(wt), _CODES[out_dtype], *args))
+    if clamped_gate_epilogue is not None:
+        return clamped_gate(y, *clamped_gate_epilogue)
     return y
 
 

@@ -81,7 +81,7 @@ class RoutedExperts(FeedForward):
     into choices, weights and gates; from there on the path is that of ``table_experts``: entries in the order of
     their experts, two grouped products, the outputs added per token in the order of its choices.  Nothing is decided
     on the host."""
-    LAUNCHES = 12
+    LAUNCHES = 11
     GRAPH_SAFE_PORTIONS = True
 
     def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, limit: float, route_scale: float = 1.0,
@@ -135,7 +135,7 @@ class RoutedExperts(FeedForward):
         choice, weights, gate = K.moe_route(logits, n, self.top, self.route_scale, self.correction,
                                             gate_col=n if self.shared_size else -1)
         eo = K.moe_order(choice, n, self.top)
-        mid = K.clamped_gate(K.moe_linear(x, self.gate_up_t, eo, from_tokens=True), self.limit, self.alpha)
+        mid = K.moe_linear(x, self.gate_up_t, eo, from_tokens=True, clamped_gate_epilogue=(self.limit, self.alpha))
         y = K.moe_linear(mid, self.down_t, eo, from_tokens=False, out_dtype=torch.float32)
         base: Optional[torch.Tensor] = None
         if self.shared_size:

@@ -110,7 +110,7 @@ def test_a_missing_key_is_named(path, key):
     (("layers", 1, "mixer", "rot", "dims"), 34, "rot.dims"), (("layers", 1, "mixer", "rot", "scaling", "high"), 0.5, "high"),
     (("layers", 0, "mlp", "router", "top"), 6, "router.top"), (("layers", 1, "mlp", "kind"), "gated", "kind"),
     (("layers", 2, "weights_of"), 2, "weights_of"), (("layers", 2, "weights_of"), 9, "weights_of"),
-    (("layers", 2, "weights_of"), 1, "differs"), (("layers", 1, "mixer", "heads"), 0, "heads")])
+    (("layers", 1, "mixer", "heads"), 0, "heads")])
 def test_a_value_that_cannot_be_is_refused(path, value, says):
     cfg = _with(pf.tiny_config_p(), path, value)
     if path[:2] == ("layers", 0):
@@ -119,11 +119,41 @@ def test_a_value_that_cannot_be_is_refused(path, value, says):
         FazopelConfig.from_dict(cfg)
 
 
-def test_a_layer_cannot_use_the_tensors_of_one_that_has_none():
+def test_a_chain_of_layers_ends_at_the_one_with_tensors():
     cfg = pf.tiny_config_p()
-    cfg["layers"].append(dict(copy.deepcopy(cfg["layers"][0]), weights_of=2))
-    with pytest.raises(ConfigError, match="no tensors of its own"):
+    cfg["layers"].append(dict(copy.deepcopy(cfg["layers"][0]), weights_of=2))      # 4 -> 2 -> 0
+    c = FazopelConfig.from_dict(cfg)
+    assert c.layers[4].weights_of == 0 and c.layers[2].weights_of == 0
+    m = build(cfg)
+    assert [r.layer for r in m.spec.order] == [0, 1, 0, 2, 0] and len(m.cache_slots) == 5
+    cfg["layers"][0]["weights_of"] = 4
+    with pytest.raises(ConfigError, match="circle"):
         FazopelConfig.from_dict(cfg)
+
+
+def test_a_layer_with_anothers_tensors_and_constants_of_its_own():
+    """The same tensors under another decay and another router scale: parts of its own that ask for layer 0's tensors."""
+    cfg = pf.tiny_config_p()
+    cfg["layers"][2]["mixer"] = dict(cfg["layers"][2]["mixer"], decay=[0.1, 0.2, 0.3])
+    cfg["layers"][2]["mlp"] = copy.deepcopy(cfg["layers"][2]["mlp"])
+    cfg["layers"][2]["mlp"]["router"]["scale"] = 3.0
+    m = build(cfg)
+    assert [r.layer for r in m.spec.order] == [0, 1, 3, 2] and len(m.spec.layers) == 4
+    assert m.spec.layers[3].parts["mixer"].params["decay"] == (0.1, 0.2, 0.3)
+    assert m.spec.layers[3].parts["ffn"].params["route_scale"] == 3.0
+    assert m.spec.layers[3].parts["mixer"].weights["q"] == "l0.mix.q" and m.spec.layers[3].parts["ffn_norm"].weights["weight"] == "l0.norm2"
+    assert {k: tuple(v.shape) for k, v in m.tensor_requests().items()} == pf.tensor_shapes(pf.tiny_config_p())
+
+
+def test_what_may_go_unsaid():
+    cfg = pf.tiny_config_p()
+    del cfg["layers"][1]["mixer"]["vdim"]                       # the attention's values are its keys
+    cfg["layers"][0]["mixer"]["decay"] = 0.75                   # one decay for all heads
+    cfg["layers"][2] = dict(copy.deepcopy(cfg["layers"][0]), weights_of=0)
+    del cfg["layers"][3]["mlp"]                                 # no feed-forward: null or absent
+    c = FazopelConfig.from_dict(cfg)
+    assert c.layers[0].mixer.decay == (0.75, 0.75, 0.75) and c.layers[3].mlp is None
+    assert build(cfg).cache_slots[1].spec == KVCacheSpec(2, 32, 0)
 
 
 def test_long_wavelengths_are_slowed_down():

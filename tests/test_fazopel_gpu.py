@@ -289,6 +289,19 @@ def test_attention_with_a_sink(gpu, dtype, sink, nh, nkv, hd, page):
 
 
 # ---- experts -------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 5, 64), (16, 65, 2048), (17, 65, 2048), (100, 13, 200), (300, 130, 96), (33, 257, 64),
+                                   (70, 9, 52), (2048, 65, 512)])
+def test_a_product_of_few_columns_with_a_32_bit_result(gpu, dtype, m, n, k):
+    """A router's scores: sums and result in 32-bit at any number of rows (few rows, many rows, rows of no whole
+    16-byte pieces, more columns than the matrix-core kernel takes)."""
+    from prelude_amd.ops import kernels as K
+    x, w = rnd((m, k), 44, dtype), rnd((n, k), 45, dtype)
+    got = K.linear_narrow_f32(x.to(gpu), w.to(gpu))
+    assert got.dtype == torch.float32
+    close(got, x.double() @ w.double().T, "float32", "scores", scale=float((x.double().abs() @ w.double().abs().T).max()))
+
+
 @pytest.mark.parametrize("E,top,T", [(5, 2, 40), (8, 3, 7), (3, 3, 19), (4, 1, 300), (70, 6, 33), (130, 8, 5)])
 def test_the_router_alone(gpu, E, top, T):
     from prelude_amd.ops import kernels as K
