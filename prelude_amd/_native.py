@@ -93,7 +93,8 @@ _KERNEL_API = {
     "pa_attn_generic_sink": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P]),
     "pa_rmsnorm_branch": (I, [P, I, P, P, I, c_long, P, P, P, I, I, F]),
     "pa_gated_rmsnorm": (I, [P, I, P, P, c_long, P, P, I, I, F]),
-    "pa_lightning_attn": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I]),
+    "pa_lightning_attn": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I]),
+    "pa_lightning_step": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, I, I, I, I, I]),
     "pa_lightning_attn_workspace": (c_long, [I, I, I, I, I, I]),
     "pa_lightning_attn_chunked": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I]),
     "pa_argmax_scratch": (I, [I, I]),

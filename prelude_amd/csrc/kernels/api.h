@@ -211,8 +211,13 @@ int pa_gated_rmsnorm(void* stream, int dtype, const float* o, const void* gate, 
 // vdim] 32-bit; sequence s owns rows cu_q[s] .. cu_q[s + 1] and slot state_slots[s]; out [tokens, heads, vdim] 32-bit.
 int pa_lightning_attn(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off, const float* decay,
                       float* state, const int* state_slots, const int* cu_q, float* out, int nseq, int tokens, int heads,
-                      int dim, int vdim, int act, int max_len);
-// max_len > 0 above: sequences of more tokens are left alone, for the call below.  The sequences seq_ids[0 .. nlisted)
+                      int dim, int vdim, int act, int max_len, int min_len);
+// The same for the step's sequences of exactly one token (a small kernel for decode steps; the same bits); with
+// min_len 2 above the two together cover a step.
+int pa_lightning_step(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off, const float* decay,
+                      float* state, const int* state_slots, const int* cu_q, float* out, int nseq, int heads, int dim,
+                      int vdim, int act);
+// max_len > 0 above: sequences of more tokens are left alone, for the call below (min_len: shorter ones too).  The sequences seq_ids[0 .. nlisted)
 // with more than `chunk` tokens (a multiple of 16 up to 256; at most max_len each) in chunks that the whole chip
 // works on at once: three passes (each chunk from a zero state, the states chained in order, what came before a chunk
 // added).  work: pa_lightning_attn_workspace(...) 32-bit words.

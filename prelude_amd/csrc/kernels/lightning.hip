@@ -55,7 +55,8 @@ enum LaMode : int { kLaWhole = 0, kLaLocal = 1, kLaApply = 2 };
 __device__ __forceinline__ size_t la_chunk_index(int row0, int chunk, int z, int j) { return (size_t)(row0 / chunk + z + j); }
 
 // R: rows of the state a lane keeps (dim <= 4 R, R a multiple of 4); NC: columns a lane keeps (64 apart).
-// kLaWhole: grid (column tiles, heads, sequences); sequences longer than `max_len` tokens (> 0) are left alone.
+// kLaWhole: grid (column tiles, heads, sequences); sequences longer than `max_len` tokens (> 0) or shorter than
+// `min_len` are left alone.
 // kLaLocal / kLaApply: grid (column tiles, heads, listed sequences x max_chunks); sequences of at most one chunk and
 // chunks past a sequence's end leave at once.
 template <typename T, int R, int NC, int MODE>
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(kLaThreads, 2) void lightning_attn_kernel(
     const T* __restrict__ qkv, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_q,
     const int* __restrict__ seq_ids, float* __restrict__ out, float* __restrict__ work, int heads, int dim, int vdim, int act,
-    int max_len, int chunk, int max_chunks) {
+    int max_len, int chunk, int max_chunks, int min_len) {
   constexpr int kCols = kLaLanes * NC;
   // a quarter's rows lie R + 4 floats apart: the four 16-byte reads of a wavefront (one a quarter) then fall into
   // different banks (R is a multiple of 8, so R floats apart they would all fall into the same four)
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(kLaThreads, 2) void lightning_attn_kernel(
   int row0 = cu_q[seq], row1 = cu_q[seq + 1];
   const int slot = state_slots[seq];
   if (slot < 0 || row1 <= row0) return;   // the same for the whole workgroup
-  if (MODE == kLaWhole && max_len > 0 && row1 - row0 > max_len) return;
+  if (MODE == kLaWhole && ((max_len > 0 && row1 - row0 > max_len) || row1 - row0 < min_len)) return;
   float* sp;
   if (MODE == kLaWhole) {
     sp = state + (((size_t)slot * heads + h) * dim) * vdim;
@@ -107,10 +108,18 @@ __global__ __launch_bounds__(kLaThreads, 2) void lightning_attn_kernel(
   for (int c = 0; c < NC; ++c) {
     col[c] = c0 + kLaLanes * c + cl;
     live[c] = col[c] < vdim;
+    // every load is unconditional (rows and columns that do not exist are clamped to ones that do, and zeroed by a
+    // select): loads under branches are waited for one by one
+    const int cc = live[c] ? col[c] : vdim - 1;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int d = dp * R + r;
-      S[c][r] = (MODE != kLaLocal && live[c] && d < dim) ? sp[(size_t)d * vdim + col[c]] : 0.f;
+      if (MODE == kLaLocal) {
+        S[c][r] = 0.f;
+      } else {
+        const float v = sp[(size_t)(d < dim ? d : dim - 1) * vdim + cc];
+        S[c][r] = (live[c] && d < dim) ? v : 0.f;
+      }
     }
   }
   // A block of sixteen tokens on its way from memory: element e of the block is token e / kPerToken's query row d,
@@ -124,18 +133,16 @@ __global__ __launch_bounds__(kLaThreads, 2) void lightning_attn_kernel(
     for (int i = 0; i < kRaw; ++i) {
       const int e = threadIdx.x + kLaThreads * i;
       const int t = e / kPerToken, x = e % kPerToken;
-      T v = from_f32<T>(0.f);   // rows past dim, columns past vdim and tokens past the end are zeros: they leave the sums alone
-      if (t0 + t < row1 && t < kLaTokens) {
-        const T* src = qkv + (size_t)(t0 + t) * ld;
-        if (x < 4 * R) {
-          if (x < dim) v = src[q_off + (size_t)h * dim + x];
-        } else if (x < 8 * R) {
-          if (x - 4 * R < dim) v = src[k_off + (size_t)h * dim + x - 4 * R];
-        } else if (c0 + x - 8 * R < vdim) {
-          v = src[v_off + (size_t)h * vdim + c0 + x - 8 * R];
-        }
-      }
-      raw[i] = v;
+      // rows past dim, columns past vdim and tokens past the end are zeros (they leave the sums alone); their loads
+      // are clamped to places that exist, so that none stands under a branch
+      const int tt = t0 + t < row1 ? t0 + t : row1 - 1;
+      const int part = x < 4 * R ? 0 : (x < 8 * R ? 1 : 2);
+      const int idx = x - (part == 0 ? 0 : (part == 1 ? 4 * R : 8 * R));
+      const int width = part == 2 ? vdim : dim;
+      const int at = part == 2 ? c0 + idx : idx;
+      const size_t base = part == 0 ? (size_t)q_off + (size_t)h * dim : (part == 1 ? (size_t)k_off + (size_t)h * dim : (size_t)v_off + (size_t)h * vdim);
+      const T v = qkv[(size_t)tt * ld + base + (at < width ? at : width - 1)];
+      raw[i] = (t0 + t < row1 && t < kLaTokens && at < width) ? v : from_f32<T>(0.f);
     }
   };
   auto stage = [&]() {
@@ -227,6 +234,58 @@ __global__ __launch_bounds__(kLaThreads, 2) void lightning_attn_kernel(
   }
 }
 
+// Sequences of exactly one token (a decode step): the same sums as the kernel above gives for them, bit for bit, in a
+// kernel small enough that a step's many launches do not wait for its code.  Grid (tiles of 64 columns, heads,
+// sequences); a wavefront owns a quarter of the rows (the quarters of the kernel above), a lane a column: a row's 64
+// columns are one run of memory.  All of a lane's rows of S are asked for at once, updated and stored; the quarters'
+// dot products meet in LDS and are added (0 + 1) + (2 + 3).
+template <typename T, int R>
+__global__ __launch_bounds__(kLaThreads) void lightning_step_kernel(
+    const T* __restrict__ qkv, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
+    float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_q, float* __restrict__ out,
+    int heads, int dim, int vdim, int act) {
+  __shared__ float qs[4 * R], ks[4 * R];
+  __shared__ float part[4][kLaLanes];
+  const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int h = blockIdx.y, seq = blockIdx.z;
+  const int row = cu_q[seq];
+  const int slot = state_slots[seq];
+  if (slot < 0 || cu_q[seq + 1] - row != 1) return;   // the same for the whole workgroup
+  const int col = blockIdx.x * kLaLanes + lane;
+  const bool live = col < vdim;
+  float* sp = state + (((size_t)slot * heads + h) * dim) * vdim + (live ? col : vdim - 1);
+  float s[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = w * R + r;
+    s[r] = sp[(size_t)(d < dim ? d : dim - 1) * vdim];
+  }
+  const T* src = qkv + (size_t)row * ld;
+  if ((int)threadIdx.x < 4 * R) {
+    const int d = (int)threadIdx.x < dim ? threadIdx.x : dim - 1;
+    qs[threadIdx.x] = la_act(to_f32(src[q_off + (size_t)h * dim + d]), act);
+    ks[threadIdx.x] = la_act(to_f32(src[k_off + (size_t)h * dim + d]), act);
+  }
+  const float v = la_act(to_f32(src[v_off + (size_t)h * vdim + (live ? col : vdim - 1)]), act);
+  const float a = decay[h];
+  __syncthreads();
+  float acc = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = w * R + r;
+    s[r] = fmaf(a, s[r], ks[d] * v);
+    if (d < dim) acc = fmaf(s[r], qs[d], acc);
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = w * R + r;
+    if (live && d < dim) sp[(size_t)d * vdim] = s[r];
+  }
+  part[w][lane] = acc;
+  __syncthreads();
+  if (w == 0 && live) out[((size_t)row * heads + h) * vdim + col] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+}
+
 // The chunks of one listed sequence in order: work[chunk] holds U coming in and the state before the chunk going
 // out; the state slot gives the start and receives the end.  A thread an element of a head's state.
 __global__ __launch_bounds__(256) void lightning_scan_kernel(const float* __restrict__ decay, float* __restrict__ state,
@@ -259,14 +318,16 @@ template <typename T, int MODE>
 static void launch_lightning(hipStream_t st, int zdim, const T* qkv, long ld, int q_off, int k_off, int v_off,
                              const float* decay, float* state, const int* state_slots, const int* cu_q, const int* seq_ids,
                              float* out, float* work, int heads, int dim, int vdim, int act, int max_len, int chunk,
-                             int max_chunks) {
+                             int max_chunks, int min_len = 0) {
   // two columns a lane where the state is wide enough and its rows leave the registers for them
-  const bool two = vdim > kLaLanes && dim <= 128;
+  // ... and there are workgroups enough without halving the columns of each (a step of few single tokens wants the
+  // workgroups)
+  const bool two = vdim > kLaLanes && dim <= 128 && (long)zdim * heads * ((vdim + 2 * kLaLanes - 1) / (2 * kLaLanes)) >= 256;
   const int cols = two ? 2 * kLaLanes : kLaLanes;
   dim3 grid((vdim + cols - 1) / cols, heads, zdim);
 #define PA_LA(R, NC)                                                                                                       \
   hipLaunchKernelGGL((lightning_attn_kernel<T, R, NC, MODE>), grid, dim3(kLaThreads), 0, st, qkv, ld, q_off, k_off, v_off, \
-                     decay, state, state_slots, cu_q, seq_ids, out, work, heads, dim, vdim, act, max_len, chunk, max_chunks)
+                     decay, state, state_slots, cu_q, seq_ids, out, work, heads, dim, vdim, act, max_len, chunk, max_chunks, min_len)
   if (dim <= 32) { if (two) PA_LA(8, 2); else PA_LA(8, 1); }
   else if (dim <= 64) { if (two) PA_LA(16, 2); else PA_LA(16, 1); }
   else if (dim <= 128) { if (two) PA_LA(32, 2); else PA_LA(32, 1); }
@@ -289,23 +350,54 @@ static int lightning_check(const char* what, int nseq, int tokens, int heads, in
 
 using namespace pa;
 
-// max_len > 0: sequences of more tokens are left alone (they go to pa_lightning_attn_chunked).
+// max_len > 0: sequences of more tokens are left alone (they go to pa_lightning_attn_chunked); sequences of fewer
+// than min_len tokens are left alone too (single tokens go to pa_lightning_step).
 extern "C" int pa_lightning_attn(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off,
                                  const float* decay, float* state, const int* state_slots, const int* cu_q, float* out,
-                                 int nseq, int tokens, int heads, int dim, int vdim, int act, int max_len) {
+                                 int nseq, int tokens, int heads, int dim, int vdim, int act, int max_len, int min_len) {
   if (nseq == 0 || tokens == 0) return 0;
   if (int rc = lightning_check("lightning_attn", nseq, tokens, heads, dim, vdim, ld, q_off, k_off, v_off, act)) return rc;
   PA_REQUIRE(nseq <= 65535, "lightning_attn: %d sequences exceed the grid", nseq);
   hipStream_t st = (hipStream_t)stream;
   if (dtype == kF32)
     launch_lightning<float, kLaWhole>(st, nseq, (const float*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
-                                      nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1);
+                                      nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1, min_len);
   else if (dtype == kBF16)
     launch_lightning<bf16, kLaWhole>(st, nseq, (const bf16*)qkv, ld, q_off, k_off, v_off, decay, state, state_slots, cu_q,
-                                     nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1);
+                                     nullptr, out, nullptr, heads, dim, vdim, act, max_len, 0, 1, min_len);
   else
     return pa::fail("lightning_attn: unknown element type code %d", dtype);
   return check_launch("lightning_attn");
+}
+
+// The sequences of exactly one token among the step's nseq (the others are left alone).
+extern "C" int pa_lightning_step(void* stream, int dtype, const void* qkv, long ld, int q_off, int k_off, int v_off,
+                                 const float* decay, float* state, const int* state_slots, const int* cu_q, float* out,
+                                 int nseq, int heads, int dim, int vdim, int act) {
+  if (nseq == 0) return 0;
+  if (int rc = lightning_check("lightning_step", nseq, nseq, heads, dim, vdim, ld, q_off, k_off, v_off, act)) return rc;
+  PA_REQUIRE(nseq <= 65535, "lightning_step: %d sequences exceed the grid", nseq);
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((vdim + kLaLanes - 1) / kLaLanes, heads, nseq);
+#define PA_LS(T, R)                                                                                                       \
+  hipLaunchKernelGGL((lightning_step_kernel<T, R>), grid, dim3(kLaThreads), 0, st, (const T*)qkv, ld, q_off, k_off, v_off, \
+                     decay, state, state_slots, cu_q, out, heads, dim, vdim, act)
+#define PA_LS_R(T)                    \
+  do {                                \
+    if (dim <= 32) PA_LS(T, 8);       \
+    else if (dim <= 64) PA_LS(T, 16); \
+    else if (dim <= 128) PA_LS(T, 32); \
+    else PA_LS(T, 64);                \
+  } while (0)
+  if (dtype == kF32)
+    PA_LS_R(float);
+  else if (dtype == kBF16)
+    PA_LS_R(bf16);
+  else
+    return pa::fail("lightning_step: unknown element type code %d", dtype);
+#undef PA_LS_R
+#undef PA_LS
+  return check_launch("lightning_step");
 }
 
 // 32-bit words of workspace for the listed sequences' chunk states

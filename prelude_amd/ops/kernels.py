@@ -1196,8 +1196,13 @@ def lightning_attention(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, d
     args = (_code(qkv), _ptr(qkv), qkv.shape[1], int(q_off), int(k_off), int(v_off), _ptr(decay), _ptr(state),
             _ptr(step.state_slots), _ptr(step.cu_q))
     act = LIGHTNING_ACTIVATIONS[activation]
-    check(kernels().pa_lightning_attn(_stream(), *args, _ptr(out), step.num_seqs, t, heads, dim, vdim, act,
-                                      int(chunk) if chunked else 0))
+    # single tokens (decode) have a small kernel of their own; the portions go to the general one
+    singles = getattr(step, "n_decode", 0) > 0
+    if singles:
+        check(kernels().pa_lightning_step(_stream(), *args, _ptr(out), step.num_seqs, heads, dim, vdim, act))
+    if step.n_prefill > 0 or not singles:
+        check(kernels().pa_lightning_attn(_stream(), *args, _ptr(out), step.num_seqs, t, heads, dim, vdim, act,
+                                          int(chunk) if chunked else 0, 2 if singles else 0))
     if chunked:
         words = kernels().pa_lightning_attn_workspace(step.n_prefill, t, heads, dim, vdim, int(chunk))
         work = torch.empty((max(words, 1),), dtype=torch.float32, device=qkv.device)

@@ -94,13 +94,15 @@ def test_unit_rms_scaled_and_gated(gpu, dtype, width):
 
 
 # ---- the recurrent mixer's kernel ---------------------------------------------------------------------------------
-def _step_of(lengths, slots, gpu):
-    """What the recurrence reads of a step: packed rows, slots, and the sequences of more than one token."""
+def _step_of(lengths, slots, gpu, singles_apart=True):
+    """What the recurrence reads of a step: packed rows, slots, and the sequences of more than one token.
+    ``singles_apart`` false: the step does not say how many single tokens it has, and they go the portions' way."""
     cu = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
     pre = [i for i, n in enumerate(lengths) if n > 1]
     return types.SimpleNamespace(
         num_seqs=len(lengths), cu_q=torch.tensor(cu, device=gpu), state_slots=torch.tensor(slots, dtype=torch.int32, device=gpu),
         prefill_seqs=torch.tensor(pre, dtype=torch.int32, device=gpu), n_prefill=len(pre),
+        n_decode=(len(lengths) - len(pre)) if singles_apart else 0,
         max_prefill_q=max([lengths[i] for i in pre], default=0))
 
 
@@ -155,11 +157,12 @@ def test_the_recurrence_does_not_depend_on_the_cut_in_32_bit(gpu):
     x = rnd((n, 2 * H * d + H * vd), 13, "float32")
     dec = torch.tensor([0.9, 0.99], device=gpu)
     outs = []
-    for cuts in ([n], [1] * n, [7, 2, 30, 1, 35]):
+    for cuts, apart in (([n], True), ([1] * n, True), ([1] * n, False), ([7, 2, 30, 1, 35], True)):   # (single tokens: both kernels)
         state = torch.zeros((1, H, d, vd), device=gpu)
         got, row = [], 0
         for c in cuts:
-            got.append(K.lightning_attention(x[row:row + c].to(gpu), 0, H * d, 2 * H * d, dec, state, _step_of([c], [0], gpu), H, d, vd))
+            got.append(K.lightning_attention(x[row:row + c].to(gpu), 0, H * d, 2 * H * d, dec, state,
+                                             _step_of([c], [0], gpu, apart), H, d, vd))
             row += c
         outs.append((torch.cat(got).cpu(), state.cpu()))
     for o, s in outs[1:]:
