@@ -215,20 +215,43 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const TX* __restrict__ 
 
 // out[t, i] = base[t, i] + sum_j weight * y[place[t * top + j], i], in ascending j; `weights` per entry, or the
 // same `weight` for all when it is null.
+constexpr int kCombineTop = 64;   // choices a token whose places and weights are staged in LDS
+
+// grid (tokens, slices of 1,024 columns): a thread adds up four columns 256 apart.  A token's places and weights are
+// read once into LDS (up to kCombineTop choices; beyond that every thread reads them as it goes).
 template <typename T>
-__global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const float* __restrict__ weights,
-                                   float weight, const T* __restrict__ base, const float* __restrict__ base_scale,
-                                   T* __restrict__ out, int top, int width) {
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place,
+                                                         const float* __restrict__ weights, float weight,
+                                                         const T* __restrict__ base, const float* __restrict__ base_scale,
+                                                         T* __restrict__ out, int top, int width) {
+  __shared__ int place_s[kCombineTop];
+  __shared__ float weight_s[kCombineTop];
   const int t = blockIdx.x;
+  const bool staged = top <= kCombineTop;
+  if (staged && (int)threadIdx.x < top) {
+    place_s[threadIdx.x] = place[t * top + threadIdx.x];
+    weight_s[threadIdx.x] = weights ? weights[t * top + threadIdx.x] : weight;
+  }
+  __syncthreads();
   const float bs = base_scale ? base_scale[t] : 1.0f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    float s = 0.f;
-    for (int j = 0; j < top; ++j) {
-      const int e = t * top + j;
-      s += (weights ? weights[e] : weight) * y[(size_t)place[e] * width + i];
+  const int i0 = blockIdx.y * 1024 + threadIdx.x;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < top; ++j) {
+    const size_t row = (size_t)(staged ? place_s[j] : place[t * top + j]) * width;
+    const float w = staged ? weight_s[j] : (weights ? weights[t * top + j] : weight);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int i = i0 + 256 * c;
+      s[c] += w * y[row + (i < width ? i : width - 1)];
     }
-    if (base) s += base_scale ? bs * to_f32(base[(size_t)t * width + i]) : to_f32(base[(size_t)t * width + i]);
-    out[(size_t)t * width + i] = from_f32<T>(s);
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int i = i0 + 256 * c;
+    if (i >= width) continue;
+    float v = s[c];
+    if (base) v += base_scale ? bs * to_f32(base[(size_t)t * width + i]) : to_f32(base[(size_t)t * width + i]);
+    out[(size_t)t * width + i] = from_f32<T>(v);
   }
 }
 
@@ -296,10 +319,10 @@ extern "C" int pa_moe_combine(void* stream, int dtype, const float* y, const int
   PA_REQUIRE(tokens > 0 && top > 0 && width > 0, "moe_combine: bad sizes tokens=%d top=%d width=%d", tokens, top, width);
   hipStream_t st = (hipStream_t)stream;
   if (dtype == kF32)
-    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(tokens), dim3(256), 0, st, y, place, weights, weight, (const float*)base,
+    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(tokens, (width + 1023) / 1024), dim3(256), 0, st, y, place, weights, weight, (const float*)base,
                        base_scale, (float*)out, top, width);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(tokens), dim3(256), 0, st, y, place, weights, weight, (const bf16*)base,
+    hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(tokens, (width + 1023) / 1024), dim3(256), 0, st, y, place, weights, weight, (const bf16*)base,
                        base_scale, (bf16*)out, top, width);
   else
     return pa::fail("moe_combine: unknown element type code %d", dtype);

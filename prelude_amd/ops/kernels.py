@@ -1366,7 +1366,8 @@ def moe_choices_by_table(token_ids: torch.Tensor, table: torch.Tensor, experts: 
 
 
 NARROW_MAX_COLUMNS = 256
-NARROW_FEW_ROWS = 16     # up to here the weight-streaming product (32-bit result from its own sums) is the faster one
+NARROW_FEW_ROWS = 64     # up to here (all it takes) the weight-streaming product, 32-bit result from its own sums: it puts
+#                          the whole chip on the weight where the kernel for narrow outputs has a workgroup per 16 rows
 
 
 def linear_narrow_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
