@@ -194,7 +194,7 @@ def test_a_token_far_back_shows_through_the_state(gpu, dtype, chunk):
 
 # ---- attention: rotation from frequencies, keys for values, a sink ------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv,hd,rot", [(4, 2, 32, 16), (6, 3, 16, 16), (1, 1, 24, 24), (4, 1, 64, 32), (8, 2, 96, 48), (2, 2, 128, 0)])
+@pytest.mark.parametrize("nh,nkv,hd,rot", [(4, 2, 32, 16), (6, 3, 16, 16), (1, 1, 24, 24), (4, 1, 64, 32), (8, 4, 96, 32), (2, 2, 128, 0)])
 def test_rotation_from_frequencies_with_the_keys_cached_as_values(gpu, dtype, nh, nkv, hd, rot):
     from prelude_amd.ops import kernels as K
     T, page, pages, eps = 9, 8, 5, 1e-5
@@ -324,7 +324,7 @@ def test_the_router_alone(gpu, E, top, T):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("E,top,T,ff,shared", [(5, 2, 50, 24, 40), (8, 3, 1, 16, 0), (3, 3, 33, 8, 8), (4, 1, 300, 32, 24), (12, 4, 400, 64, 128)])
+@pytest.mark.parametrize("E,top,T,ff,shared", [(5, 2, 50, 24, 40), (8, 3, 1, 16, 0), (3, 3, 33, 8, 8), (4, 1, 300, 32, 24), (10, 4, 400, 48, 96)])
 def test_routed_experts(gpu, dtype, E, top, T, ff, shared):
     """The part alone on the numbers the plain one gets (so both routers see the same scores): unequal loads, an
     expert nobody chooses, every expert chosen, one token, more tokens than a tile."""
