@@ -425,6 +425,31 @@ def test_every_layer_of_the_stream(gpu):
         close(a, b, "float32", f"after layer run {i}")
 
 
+def test_a_layer_with_anothers_tensors_under_constants_of_its_own(gpu):
+    """A layer that names another's tensors but has another decay, router scale and clamp: the engine runs layer 0's
+    tensors under that entry's constants, in portions and single tokens, as the plain implementation does."""
+    from prelude_amd.trace import TraceRunner
+    from prelude_amd.weights import write_safetensors
+    cfg = pf.tiny_config_p()
+    cfg["layers"][2] = json.loads(json.dumps(cfg["layers"][2]))
+    cfg["layers"][2]["mixer"]["decay"] = [0.2, 0.97, 0.6]
+    cfg["layers"][2]["mlp"]["router"]["scale"] = 0.5
+    cfg["layers"][2]["mlp"]["expert"]["limit"] = 0.4
+    w = pf.random_weights(cfg, 21)
+    toks = torch.randint(0, cfg["vocab"], (90,), generator=torch.Generator().manual_seed(5)).tolist()
+    ref = pf.forward(cfg, w, toks)
+    same = pf.tiny_config_p()
+    assert float((pf.forward(same, w, toks) - ref).abs().max()) > 0.3 * float(ref.std()), "the constants matter"
+    with tempfile.TemporaryDirectory(prefix="prelude_amd_fazopel_own_") as d:
+        with open(os.path.join(d, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        write_safetensors(os.path.join(d, "model.safetensors"), {k: v.to(torch.bfloat16) for k, v in w.items()})
+        r = TraceRunner(d, "float32", 128, page_size=8, state_slots=1)
+        outs = [r.step([{"id": 0, "tokens": toks[:70], "want": list(range(70))}])]
+        outs += [r.step([{"id": 0, "tokens": [t], "want": [0]}]) for t in toks[70:]]
+    check(np.concatenate(outs), ref, "float32", "constants of its own")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["p", "q", "r"])
 def test_prefill_then_token_by_token(gpu, name, dtype):
