@@ -47,9 +47,11 @@ class RotaryFrequencies(PositionEncoding):
 
     def __init__(self, rotary_dim: int, theta: float, long_wave_factor: float = 0.0, long_wave_low: float = 1.0,
                  long_wave_high: float = 1.0, long_wave_original: int = 0):
-        """``long_wave_factor`` > 0 slows the long wavelengths down, by wavelength l = 2 pi / f against a length
-        ``long_wave_original``: l < original / high keeps f; l > original / low takes f / factor; between them,
-        with s = (original / l - low) / (high - low), (1 - s) f / factor + s f.  0: the plain frequencies."""
+        """``long_wave_factor`` > 0 slows the long wavelengths down.  With lambda = 2 pi / f a frequency's wavelength,
+        lambda_short = ``long_wave_original`` / ``long_wave_high`` and lambda_long = ``long_wave_original`` /
+        ``long_wave_low``: waves shorter than lambda_short keep f, waves longer than lambda_long turn at f / factor,
+        and those between move from the one to the other, f / factor + t (f - f / factor) with
+        t = (original / lambda - low) / (high - low).  0: the plain frequencies."""
         if rotary_dim <= 0 or rotary_dim % 2:
             raise PartError(f"rotary_frequencies: rotary width {rotary_dim} must be positive and even")
         if theta <= 0:

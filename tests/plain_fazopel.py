@@ -44,9 +44,9 @@ def decaying_state_mixer(h, w, pre, m, eps, state=None):
 
 # ---- attention ---------------------------------------------------------------------------------------------------
 def scaled_frequencies(rot, dtype=torch.float64):
-    """f_i = base^(-2i/dims), then long wavelengths slowed down: wavelength l = 2 pi / f; l < original / high keeps
-    f, l > original / low gives f / factor, and between them the two are blended by
-    s = (original / l - low) / (high - low): (1 - s) f / factor + s f."""
+    """f_i = base^(-2i/dims); with a scaling, by each frequency's wavelength lambda = 2 pi / f_i: short waves
+    (lambda < original / high) keep f_i, long ones (lambda > original / low) get f_i / factor, and a wave between the
+    two a mixture of both, weighted t and 1 - t with t = (original / lambda - low) / (high - low)."""
     dims = rot["dims"]
     f = torch.tensor([float(rot["base"]) ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=dtype)
     sc = rot.get("scaling")
